@@ -1,0 +1,209 @@
+/*
+ * iris_amd.h -- C-ABI of the MI355X-native fused GEMM + tile-publishing path.
+ *
+ * Two shared libraries implement it:
+ *
+ *   libfinegrained_allocator.so   torch pluggable-allocator entry points
+ *   libiris_amd.so                HIP runtime helpers + kernel launchers
+ *
+ * Everything is `extern "C"`, takes plain pointers and integers, allocates
+ * nothing (except the two allocator calls whose job that is), never
+ * synchronises the stream and never takes ownership of a buffer.  A HIP
+ * stream is passed as `void*` (a `hipStream_t`); NULL is the default stream.
+ * Unless stated otherwise a function returns a `hipError_t` as `int`
+ * (0 == hipSuccess); `iris_hip_error_string` turns it into text.
+ *
+ * Reference citations are relative to the ROCm/iris tree.
+ */
+#ifndef IRIS_AMD_H_
+#define IRIS_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+#include <sys/types.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------ */
+/* Pluggable allocator (libfinegrained_allocator.so)                         */
+/* Replaces csrc/finegrained_alloc/finegrained_allocator.hip:28-55, bound by */
+/* torch.cuda.memory.CUDAPluggableAllocator at iris/__init__.py:40-45.       */
+/* On a HIP error both print "[finegrained_allocator] Hip error: ..." to     */
+/* stderr and exit(EXIT_FAILURE), as the reference does (:11-16).            */
+/* ------------------------------------------------------------------------ */
+void* finegrained_hipMalloc(ssize_t size, int device, void* stream);
+void finegrained_hipFree(void* ptr, ssize_t size, int device, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* HIP runtime helpers (libiris_amd.so); replace iris/_hip.py                */
+/* ------------------------------------------------------------------------ */
+/* hipGetErrorString; iris/_hip.py:12-16 */
+const char* iris_hip_error_string(int err);
+/* iris/_hip.py:62-65 */
+int iris_hip_device_count(int* count);
+/* iris/_hip.py:68-69 */
+int iris_hip_set_device(int device);
+/* iris/_hip.py:72-75 */
+int iris_hip_get_device(int* device);
+/* hipDeviceAttributeMultiprocessorCount; iris/_hip.py:78-87 */
+int iris_hip_cu_count(int device, int* cu_count);
+/* hipDeviceAttributeWallClockRate, kHz; iris/_hip.py:107-114 */
+int iris_hip_wall_clock_rate(int device, int* khz);
+/* hipExtMallocWithFlags(hipDeviceMallocFinegrained); iris/_hip.py:117-121 */
+int iris_hip_malloc_finegrained(void** ptr, size_t size);
+/* hipMalloc / hipFree; iris/_hip.py:124-131 */
+int iris_hip_malloc(void** ptr, size_t size);
+int iris_hip_free(void* ptr);
+/* hipIpcGetMemHandle, 64-byte handle; iris/_hip.py:56-59 */
+int iris_hip_ipc_get_handle(void* handle64, void* ptr);
+/* hipIpcOpenMemHandle(..., hipIpcMemLazyEnablePeerAccess); iris/_hip.py:23-53 */
+int iris_hip_ipc_open_handle(void** ptr, const void* handle64);
+/* hipDeviceSynchronize: the device half of Iris.barrier, iris/iris.py:272-276 */
+int iris_hip_device_synchronize(void);
+/* name of the gfx target the current device reports ("gfx950"); buf gets a
+ * NUL-terminated string of at most len-1 characters */
+int iris_hip_arch_name(int device, char* buf, size_t len);
+
+/* ------------------------------------------------------------------------ */
+/* Kernel launchers (libiris_amd.so)                                         */
+/* ------------------------------------------------------------------------ */
+
+/* element types */
+#define IRIS_DTYPE_F32 0
+#define IRIS_DTYPE_F16 1
+#define IRIS_DTYPE_BF16 2
+
+/* epilogues of the persistent shard GEMM */
+#define IRIS_EPI_ALL_SCATTER 0 /* examples/07_gemm_all_scatter/gemm_all_scatter.py:209-251 */
+#define IRIS_EPI_ATOMIC_ADD 1  /* examples/08_gemm_atomics_all_reduce/gemm_atomics_all_reduce.py:206-248 */
+#define IRIS_EPI_ONE_SHOT 2    /* examples/09_gemm_one_shot_all_reduce/gemm_one_shot_all_reduce.py:197-271 */
+
+/* phases of IRIS_EPI_ONE_SHOT (bit mask) */
+#define IRIS_PHASE_PRODUCE 1 /* store partial tile + signal the other ranks  (:197-218) */
+#define IRIS_PHASE_CONSUME 2 /* wait for the tile's flag, reduce, store       (:220-271) */
+#define IRIS_PHASE_FUSED 3   /* both, in one program, as the reference kernel */
+
+/* flag scopes */
+#define IRIS_SCOPE_AGENT 0  /* all "ranks" live on this GPU */
+#define IRIS_SCOPE_SYSTEM 1 /* the reference's scope="sys" */
+
+/* status word values (max-reduced by the kernels into *status) */
+#define IRIS_STATUS_OK 0
+#define IRIS_STATUS_SPIN_TIMEOUT 1 /* a flag wait gave up; that tile was not reduced */
+
+/*
+ * Arguments of one persistent shard-GEMM launch.  It is the argument list of
+ * the reference kernels (gemm_*:95-132) plus what their Triton launch passes
+ * implicitly (element types, stream).  Strides are in elements.
+ */
+typedef struct iris_gemm_args {
+  const void* a;        /* A  [M, K]                                   gemm_*:96  */
+  const void* b;        /* B  [K, N]                                   gemm_*:97  */
+  void* c;              /* this rank's partial C [M, N] (ONE_SHOT)      gemm_*:98  */
+  void* c_global;       /* published result                            gemm_*:99  */
+  int32_t* tile_completed; /* one flag per tile, on the heap            gemm_*:103 */
+  const uint64_t* heap_bases; /* device uint64[world_size]              gemm_*:125 */
+  int64_t* mm_begin_timestamp; /* optional int64[total_tiles]           gemm_*:130 */
+  int64_t* mm_end_timestamp;   /* optional int64[total_tiles]           gemm_*:131 */
+  uint32_t* status;     /* optional device word, see IRIS_STATUS_*                */
+  int32_t M, N, K;      /*                                              gemm_*:104-106 */
+  int64_t stride_am, stride_ak; /*                                      gemm_*:107-108 */
+  int64_t stride_bk, stride_bn; /*                                      gemm_*:109-110 */
+  int64_t stride_cm, stride_cn; /*                                      gemm_*:111-112 */
+  int64_t stride_cm_global, stride_cn_global; /*                        gemm_*:113-114 */
+  int32_t block_m, block_n, block_k; /* BLOCK_SIZE_*                    gemm_*:116-118 */
+  int32_t group_size_m; /* GROUP_SIZE_M                                 gemm_*:119 */
+  int32_t num_sms;      /* NUM_SMS == grid size                         gemm_*:120 */
+  int32_t num_xcds;     /* NUM_XCDS                                     gemm_*:122 */
+  int32_t cur_rank, world_size; /*                                      gemm_*:126-127 */
+  int32_t ab_dtype;     /* IRIS_DTYPE_F16 | IRIS_DTYPE_BF16                       */
+  int32_t c_dtype;      /* element type of c                                      */
+  int32_t c_global_dtype; /* element type of c_global                             */
+  int32_t epilogue;     /* IRIS_EPI_*                                             */
+  int32_t phase;        /* IRIS_PHASE_* (ONE_SHOT only)                           */
+  int32_t notify;       /* ALL_SCATTER: publish a ready flag per tile   gemm_*:128 (NOTIFY_REMOTES) */
+  int32_t scope;        /* IRIS_SCOPE_*                                           */
+  int32_t variant;      /* 0 = default kernel choice; >0 selects a tuning variant */
+  uint64_t spin_timeout_ticks; /* bound on a flag wait in 100 MHz ticks; 0 = default (2 s) */
+} iris_gemm_args;
+
+/*
+ * Launch the persistent shard GEMM with the epilogue `args->epilogue`.
+ * Replaces `gemm_kernel[(grids,)](...)` at matmul_wrapper.py:109-150 (the same file in
+ * examples/07_gemm_all_scatter, 08_gemm_atomics_all_reduce and 09_gemm_one_shot_all_reduce).
+ * Returns hipErrorInvalidValue for shapes/strides/types it does not take.
+ */
+int iris_gemm_launch(const iris_gemm_args* args, void* stream);
+
+/* Registers and spills of the kernel `iris_gemm_launch` would pick for `args`
+ * (what the reference reads from kk.n_regs / kk.n_spills,
+ * matmul_wrapper.py:152-155).  *spills is the scratch bytes per lane. */
+int iris_gemm_kernel_info(const iris_gemm_args* args, int* n_regs, int* n_spills);
+
+/* Name of tuning variant `variant` (1-based) of the kernel list used for
+ * (ab_dtype, fp32 output?, atomic?); hipErrorInvalidValue past the end. */
+int iris_gemm_variant_name(int ab_dtype, int out_is_f32, int atomic, int variant, char* buf, size_t len);
+
+/*
+ * One-shot reduce of `world_size` partial-C buffers that live at the same
+ * heap offset on every rank: wait for tile_completed[tile] == world_size-1
+ * (CAS back to 0, acquire), sum the tile over ranks 0..world_size-1 in fp32,
+ * store to c_global.  The consumer half of
+ * examples/09_gemm_one_shot_all_reduce/gemm_one_shot_all_reduce.py:220-271
+ * as a kernel of its own.  `c` is this rank's partial buffer.
+ */
+typedef struct iris_reduce_args {
+  const void* c;
+  void* c_global;
+  int32_t* tile_completed;
+  const uint64_t* heap_bases;
+  uint32_t* status;
+  int32_t M, N;
+  int64_t stride_cm, stride_cn;
+  int64_t stride_cm_global, stride_cn_global;
+  int32_t block_m, block_n, group_size_m;
+  int32_t num_sms;   /* grid size; 0 = one program per tile */
+  int32_t num_xcds;
+  int32_t cur_rank, world_size;
+  int32_t c_dtype, c_global_dtype;
+  int32_t scope;
+  int32_t wait_flags; /* 0: skip the flag wait (plain P-way sum) */
+  int32_t variant;
+  uint64_t spin_timeout_ticks;
+} iris_reduce_args;
+
+int iris_one_shot_reduce_launch(const iris_reduce_args* args, void* stream);
+
+/*
+ * The producer's signal on its own: +1 (release) on tile_completed[tile] of
+ * every rank other than cur_rank (include_self != 0: of every rank), for
+ * tile in [0, total_tiles).  gemm_one_shot_all_reduce.py:207-218.
+ */
+int iris_signal_tiles_launch(int32_t* tile_completed, const uint64_t* heap_bases, int32_t total_tiles,
+                             int32_t cur_rank, int32_t world_size, int32_t include_self, int32_t scope,
+                             void* stream);
+
+/* int32 fill; iris/util.py:107-128 (memset_kernel / memset_tensor). */
+int iris_memset_i32_launch(int32_t* ptr, int32_t value, int64_t n_elements, void* stream);
+
+/*
+ * The tile schedule exactly as the kernels compute it, for checking it bit
+ * for bit: out is int32[total_tiles][4] = (pid_m, pid_n, program, position
+ * in the program's tile list) per tile id.  tile_id -> (pid_m, pid_n) is
+ * gemm_*:155-160; the program's tile list is gemm_*:133-136,150.
+ */
+int iris_tile_schedule_launch(int32_t* out, int32_t M, int32_t N, int32_t block_m, int32_t block_n,
+                              int32_t group_size_m, int32_t num_sms, int32_t num_xcds, void* stream);
+/* The same tile_id -> (pid_m, pid_n) function, compiled for the host. */
+void iris_tile_map_host(int32_t tile_id, int32_t M, int32_t N, int32_t block_m, int32_t block_n,
+                        int32_t group_size_m, int32_t* pid_m, int32_t* pid_n);
+
+/* Library version, bumped when a signature in this header changes. */
+int iris_amd_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IRIS_AMD_H_ */

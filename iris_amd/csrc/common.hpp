@@ -1,0 +1,163 @@
+// Shared device/host helpers for the gfx950 kernels of the fused GEMM +
+// tile-publishing path.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/iris_amd.h"
+
+namespace iris_amd {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+#define IRIS_LDS __attribute__((address_space(3)))
+// Device memory.  Pointers rebuilt from integers would otherwise be "flat",
+// and flat accesses tie the LDS counter to the vector-memory counter.
+#define IRIS_GLOBAL __attribute__((address_space(1)))
+
+// s_waitcnt immediates for gfx9-family encodings: vmcnt[3:0] in bits 3:0,
+// vmcnt[5:4] in bits 15:14, expcnt in 6:4, lgkmcnt in 11:8.  These leave
+// expcnt and lgkmcnt unconstrained.
+#define IRIS_WAIT_VMCNT(n) \
+  __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (0x7 << 4) | (0xF << 8) | ((((n) >> 4) & 0x3) << 14))
+#define IRIS_WAIT_LGKMCNT0() __builtin_amdgcn_s_waitcnt(0xC07F)
+
+struct TileCoord {
+  int pid_m;
+  int pid_n;
+};
+
+// tile_id -> (pid_m, pid_n) with the GROUP_SIZE_M swizzle; the arithmetic of
+// examples/09_gemm_one_shot_all_reduce/gemm_one_shot_all_reduce.py:155-160.
+__host__ __device__ inline TileCoord tile_map(int tile_id, int num_pid_m, int num_pid_n, int G) {
+  const int num_pid_in_group = G * num_pid_n;
+  const int group_id = tile_id / num_pid_in_group;
+  const int first_pid_m = group_id * G;
+  const int rem = num_pid_m - first_pid_m;
+  const int group_size_m = rem < G ? rem : G;
+  const int in_group = tile_id % num_pid_in_group;
+  TileCoord t;
+  t.pid_m = first_pid_m + (in_group % group_size_m);
+  t.pid_n = in_group / group_size_m;
+  return t;
+}
+
+// program-id remap that keeps consecutive tiles on one XCD;
+// gemm_one_shot_all_reduce.py:135-136.
+__host__ __device__ inline int xcd_remap(int pid, int num_sms, int num_xcds) {
+  if (num_xcds != 1) pid = (pid % num_xcds) * (num_sms / num_xcds) + (pid / num_xcds);
+  return pid;
+}
+
+// Pointer rebasing between symmetric heaps; iris/iris.py:317-339.
+template <typename P>
+__device__ inline IRIS_GLOBAL P* translate(P* ptr, uint64_t cur_base, uint64_t target_base) {
+  const uint64_t off = reinterpret_cast<uint64_t>(ptr) - cur_base;
+  return (IRIS_GLOBAL P*)(target_base + off);
+}
+
+// ---- element conversions ---------------------------------------------------
+
+__device__ inline unsigned short f32_to_bf16_bits(float f) {
+  return __builtin_bit_cast(unsigned short, (__bf16)f);  // round-to-nearest-even
+}
+__device__ inline float bf16_bits_to_f32(unsigned short h) {
+  return __builtin_bit_cast(float, ((unsigned int)h) << 16);
+}
+__device__ inline unsigned short f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;  // v_cvt_f16_f32, round-to-nearest-even
+  return __builtin_bit_cast(unsigned short, h);
+}
+__device__ inline float f16_bits_to_f32(unsigned short h) {
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+
+// to16<DT>(f): fp32 -> 16-bit pattern of element type DT (IRIS_DTYPE_*),
+// round-to-nearest-even (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32 on gfx950)
+template <int DT>
+__device__ inline unsigned int pack2(float lo, float hi) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  const f32x2 v = {lo, hi};
+  if constexpr (DT == IRIS_DTYPE_BF16)
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, bf16x2));
+  else
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, f16x2));
+}
+template <int DT>
+__device__ inline unsigned short to16(float f) {
+  return (unsigned short)(pack2<DT>(f, 0.f) & 0xFFFFu);
+}
+template <int DT>
+__device__ inline float from16(unsigned short h) {
+  if constexpr (DT == IRIS_DTYPE_BF16)
+    return bf16_bits_to_f32(h);
+  else
+    return f16_bits_to_f32(h);
+}
+
+// Bare workgroup barrier.  __syncthreads() (and any LDS release fence) also
+// drains the vector-memory counter, because LDS-DMA loads count as LDS
+// writes; that would stall on the slabs that are meant to stay in flight
+// across the barrier.  The caller waits explicitly for the one slab it needs.
+// The empty asm statements keep the compiler from moving memory accesses
+// across the barrier.
+__device__ inline void block_barrier_raw() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+__host__ __device__ inline int dtype_size(int dt) { return dt == IRIS_DTYPE_F32 ? 4 : 2; }
+
+// ---- scoped atomics on flags -----------------------------------------------
+
+__device__ inline void flag_add_release(IRIS_GLOBAL int32_t* p, int v, bool sys) {
+  if (sys)
+    __hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  else
+    __hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// CAS(expected -> desired) with acquire; returns the old value
+// (tl.atomic_cas semantics, iris/iris.py:476-497).
+__device__ inline int flag_cas_acquire(IRIS_GLOBAL int32_t* p, int expected, int desired, bool sys) {
+  int e = expected;
+  if (sys)
+    __hip_atomic_compare_exchange_strong(p, &e, desired, __ATOMIC_ACQUIRE, __ATOMIC_ACQUIRE,
+                                         __HIP_MEMORY_SCOPE_SYSTEM);
+  else
+    __hip_atomic_compare_exchange_strong(p, &e, desired, __ATOMIC_ACQUIRE, __ATOMIC_ACQUIRE,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+  return e;
+}
+
+// Bounded wait for a tile's flag: spins on CAS(ws-1 -> 0) until the old value
+// reaches ws-1 (gemm_one_shot_all_reduce.py:220-234) or `timeout` ticks of
+// the 100 MHz wall clock have passed.  Returns true on success.  Every caller
+// reaches an exit: a wait that gives up records IRIS_STATUS_SPIN_TIMEOUT.
+__device__ inline bool wait_tile_flag(IRIS_GLOBAL int32_t* flag, int ws, bool sys, uint64_t timeout,
+                                      uint32_t* status) {
+  if (ws <= 1) return true;  // `while result < ws-1` never runs for ws == 1
+  const uint64_t t0 = wall_clock64();
+  for (;;) {
+    const int old = flag_cas_acquire(flag, ws - 1, 0, sys);
+    if (old >= ws - 1) return true;
+    if (wall_clock64() - t0 > timeout) {
+      if (status) atomicMax(status, (uint32_t)IRIS_STATUS_SPIN_TIMEOUT);
+      return false;
+    }
+    __builtin_amdgcn_s_sleep(8);
+  }
+}
+
+}  // namespace iris_amd

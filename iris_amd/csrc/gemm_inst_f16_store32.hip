@@ -1,0 +1,13 @@
+// Shard-GEMM kernel instantiations: f16 operands, store32 epilogue.
+#include "gemm_registry.hpp"
+
+namespace iris_amd {
+
+static const GemmKernelEntry k_entries[] = {IRIS_GEMM_VARIANTS(IRIS_GEMM_ENTRY, IRIS_DTYPE_F16, OP_STORE32)};
+
+const GemmKernelEntry* gemm_entries_f16_store32(int* count) {
+  *count = (int)(sizeof(k_entries) / sizeof(k_entries[0]));
+  return k_entries;
+}
+
+}  // namespace iris_amd

@@ -1,0 +1,579 @@
+// Persistent shard GEMM for gfx950 (MI355X) with the three tile-publishing
+// epilogues.  One workgroup per CU walks its tiles
+// `for tile_id in range(pid, total_tiles, NUM_SMS)`
+// (examples/09_gemm_one_shot_all_reduce/gemm_one_shot_all_reduce.py:150) and,
+// for every tile, runs the K loop of :174-195 on the matrix cores:
+//
+//   * A[M,K] and B[K,N] are both K-contiguous.  A CM x BK slab of A and a
+//     CN x BK slab of B are copied HBM -> LDS with `buffer_load ... lds`
+//     (16 bytes per lane, no register staging) into an S-deep ring of stages.
+//     The ring is fed S-1 K-steps ahead and runs *across* tile boundaries, so
+//     the next tile's first slabs are already in flight during an epilogue.
+//   * LDS holds each slab row-major with the 16-byte chunks of a row XOR-ed
+//     by the row index so that the `ds_read_b128` operand fetches of one MFMA
+//     are bank-conflict free.
+//   * v_mfma_f32_32x32x16 (bf16 or f16) with fp32 accumulators; operands are
+//     swapped (B rows as SrcA, A rows as SrcB) so that a lane ends up with 4
+//     consecutive columns of one output row.
+//   * The epilogue transposes the accumulators through a wave-private LDS
+//     scratch so that global stores / atomics cover contiguous row segments.
+//
+// The logical tile (BLOCK_SIZE_M x BLOCK_SIZE_N, which fixes tile ids and
+// flags) may be larger than the compute tile (CM x CN); a logical tile is
+// then covered by several compute tiles and published once.
+#pragma once
+
+#include "common.hpp"
+
+namespace iris_amd {
+
+struct GemmKArgs {
+  const char* a;
+  const char* b;
+  char* out;  // c (ONE_SHOT producer) or c_global, already at its column offset
+  int32_t* flags;
+  const uint64_t* heap_bases;
+  int64_t* ts_begin;
+  int64_t* ts_end;
+  int64_t sam, sak, sbk, sbn;  // A/B strides, elements
+  int64_t som, son;            // strides of `out`, elements
+  int M, N, K;
+  int BM, BN, G;
+  int num_sms, num_xcds, cur_rank, ws;
+  int num_pid_m, num_pid_n, total_tiles;
+  int sub_m, sub_n;  // compute tiles per logical tile
+  int dest_all;      // write `out` on every rank's heap (else on this rank only)
+  int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
+  int sys;           // flag atomics at system scope (else agent)
+  int vec_out;       // 16-byte vector access allowed on `out`
+};
+
+template <int DT>
+struct Mfma;
+template <>
+struct Mfma<IRIS_DTYPE_BF16> {
+  using vec8 = bf16x8;
+  __device__ static inline f32x16 run(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<IRIS_DTYPE_F16> {
+  using vec8 = f16x8;
+  __device__ static inline f32x16 run(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <int DT_, int CM_, int CN_, int BK_, int WM_, int WN_, int S_, bool DMA_>
+struct GemmCfg {
+  static constexpr int DT = DT_, CM = CM_, CN = CN_, BK = BK_, WM = WM_, WN = WN_, S = S_;
+  static constexpr bool DMA = DMA_;
+  static constexpr int NW = WM * WN, NT = NW * 64;
+  static constexpr int TM = CM / WM, TN = CN / WN;
+  static constexpr int IM = TM / 32, IN = TN / 32;
+  static constexpr int CPR = BK / 8;    // 16-byte chunks per slab row
+  static constexpr int RP = 16 / CPR;   // slab rows per 256 bytes
+  static constexpr int RPB = 64 / CPR;  // slab rows per 1 KiB block (one wave-wide DMA)
+  static constexpr int A_BYTES = CM * BK * 2, B_BYTES = CN * BK * 2;
+  static constexpr int STAGE = A_BYTES + B_BYTES;
+  static constexpr int A_LOADS = CM * CPR / NT, B_LOADS = CN * CPR / NT;
+  static constexpr int L = A_LOADS + B_LOADS;
+  static constexpr int KSUB = BK / 16;
+  // wave-private epilogue scratch: 32 rows x TN 16-bit elements
+  static constexpr int WS_PITCH = TN * 2;
+  static constexpr int WS_BYTES = 32 * WS_PITCH;
+  static constexpr int U16 = TN / 8;       // 16-byte units per scratch row
+  static constexpr int ERPB = 128 / TN;    // scratch rows per 256 bytes
+  static constexpr int LDS_BYTES = S * STAGE + NW * WS_BYTES;
+  static_assert(CM % (WM * 32) == 0 && CN % (WN * 32) == 0, "wave tile must be a multiple of 32x32");
+  static_assert(BK == 32 || BK == 64, "BK");
+  static_assert((CM * CPR) % NT == 0 && (CN * CPR) % NT == 0, "slab must split evenly over lanes");
+  static_assert(A_LOADS >= 1 && B_LOADS >= 1, "too many waves for this slab");
+  static_assert((S & (S - 1)) == 0 && S >= 1, "ring depth must be a power of two");
+  static_assert(L * (S > 2 ? S - 2 : 0) <= 63, "vmcnt immediate");
+  static_assert(TN == 32 || TN == 64 || TN == 128, "wave tile width");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+};
+
+// One compute tile of work.
+struct Item {
+  int tile_id;
+  int m0, n0;        // origin of the compute tile
+  int m_end, n_end;  // exclusive bounds (logical tile clipped to M, N)
+  int lm0, ln0;      // origin of the logical tile
+  bool last_sub;     // last compute tile of its logical tile
+  bool first_sub;
+};
+
+template <class Cfg>
+__device__ inline Item decode_item(const GemmKArgs& p, int pid, int item) {
+  const int subs = p.sub_m * p.sub_n;
+  const int ti = item / subs;
+  const int s = item - ti * subs;
+  Item it;
+  it.tile_id = pid + ti * p.num_sms;
+  const TileCoord tc = tile_map(it.tile_id, p.num_pid_m, p.num_pid_n, p.G);
+  it.lm0 = tc.pid_m * p.BM;
+  it.ln0 = tc.pid_n * p.BN;
+  const int sm = s / p.sub_n, sn = s - sm * p.sub_n;
+  it.m0 = it.lm0 + sm * Cfg::CM;
+  it.n0 = it.ln0 + sn * Cfg::CN;
+  it.m_end = min(p.M, it.lm0 + p.BM);
+  it.n_end = min(p.N, it.ln0 + p.BN);
+  it.first_sub = (s == 0);
+  it.last_sub = (s == subs - 1);
+  return it;
+}
+
+// `ptr` as seen on rank r's heap (identity for the caller's own rank).
+template <typename P>
+__device__ inline IRIS_GLOBAL P* rank_ptr(const GemmKArgs& p, P* ptr, int r) {
+  if (r == p.cur_rank || p.heap_bases == nullptr) return (IRIS_GLOBAL P*)ptr;
+  return translate(ptr, p.heap_bases[p.cur_rank], p.heap_bases[r]);
+}
+
+// ---------------------------------------------------------------------------
+// Slab loader
+// ---------------------------------------------------------------------------
+
+// Per-item loader state.  Lane `lane` of wave `wave` fetches, for load `i`,
+// the 16-byte chunk that lands at byte  blk*1024 + lane*16  of the slab,
+// blk = i*NW + wave.  That position is (row, physical chunk); the chunk of the
+// row it must hold is  pc ^ ((row / RP) % CPR).
+template <class Cfg>
+struct Loader {
+  __amdgpu_buffer_rsrc_t ra, rb;
+  uint32_t voff[Cfg::L];  // byte offset of (row, logical chunk) at k0 == 0
+  uint32_t kcol[Cfg::L];  // first k of the chunk at k0 == 0
+
+  __device__ inline void setup(const GemmKArgs& p, const Item& it, int wave, int lane) {
+    // Rows past the matrix edge re-read the last valid row (the reference
+    // wraps with % M / % N, gemm_*:162-163); their results are never stored.
+    const int m0c = min(it.m0, p.M - 1), n0c = min(it.n0, p.N - 1);
+    const int rows_a = min(Cfg::CM, p.M - m0c), rows_b = min(Cfg::CN, p.N - n0c);
+    const char* abase = p.a + (int64_t)m0c * p.sam * 2;
+    const char* bbase = p.b + (int64_t)n0c * p.sbn * 2;
+    const uint32_t arec = (uint32_t)(((int64_t)(rows_a - 1) * p.sam + p.K) * 2);
+    const uint32_t brec = (uint32_t)(((int64_t)(rows_b - 1) * p.sbn + p.K) * 2);
+    ra = __builtin_amdgcn_make_buffer_rsrc((void*)abase, 0, arec, 0x00020000);
+    rb = __builtin_amdgcn_make_buffer_rsrc((void*)bbase, 0, brec, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < Cfg::L; ++i) {
+      const bool isA = i < Cfg::A_LOADS;
+      const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
+      const int row = blk * Cfg::RPB + lane / Cfg::CPR;
+      const int pc = lane % Cfg::CPR;
+      const int ch = pc ^ ((row / Cfg::RP) % Cfg::CPR);
+      const int rclamp = min(row, (isA ? rows_a : rows_b) - 1);
+      const int64_t ld = isA ? p.sam : p.sbn;
+      voff[i] = (uint32_t)(((int64_t)rclamp * ld + ch * 8) * 2);
+      kcol[i] = ch * 8;
+    }
+  }
+
+  // Issue the L loads of K-step `k` into the stage at LDS address `stage`.
+  __device__ inline void issue(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
+    const int k0 = k * Cfg::BK;
+#pragma unroll
+    for (int i = 0; i < Cfg::L; ++i) {
+      const bool isA = i < Cfg::A_LOADS;
+      const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
+      IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + blk * 1024;
+      // chunks past K read as zero: an offset beyond num_records is out of
+      // range for the buffer and the load returns 0 (the masked tail of
+      // gemm_*:186-195)
+      const uint32_t off = ((int)(k0 + kcol[i]) < p.K) ? voff[i] + (uint32_t)k0 * 2 : 0x80000000u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, 0, 0, 0);
+    }
+  }
+};
+
+// Generic loader: any strides / alignment, element by element, synchronous.
+// It writes the same slab layout.
+template <class Cfg>
+__device__ inline void load_slab_generic(const GemmKArgs& p, const Item& it, IRIS_LDS char* stage, int k,
+                                         int tid) {
+  const int k0 = k * Cfg::BK;
+  const IRIS_GLOBAL unsigned short* A = (const IRIS_GLOBAL unsigned short*)p.a;
+  const IRIS_GLOBAL unsigned short* B = (const IRIS_GLOBAL unsigned short*)p.b;
+  for (int idx = tid; idx < (Cfg::CM + Cfg::CN) * Cfg::CPR; idx += Cfg::NT) {
+    const bool isA = idx < Cfg::CM * Cfg::CPR;
+    const int pos = isA ? idx : idx - Cfg::CM * Cfg::CPR;
+    const int row = pos / Cfg::CPR, pc = pos % Cfg::CPR;
+    const int ch = pc ^ ((row / Cfg::RP) % Cfg::CPR);
+    u32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      unsigned int w = 0;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int kk = k0 + ch * 8 + e * 2 + h;
+        unsigned short x = 0;
+        if (kk < p.K) {
+          if (isA) {
+            const int r = min(it.m0 + row, p.M - 1);
+            x = A[(int64_t)r * p.sam + (int64_t)kk * p.sak];
+          } else {
+            const int r = min(it.n0 + row, p.N - 1);
+            x = B[(int64_t)r * p.sbn + (int64_t)kk * p.sbk];
+          }
+        }
+        w |= ((unsigned int)x) << (16 * h);
+      }
+      v[e] = w;
+    }
+    *reinterpret_cast<IRIS_LDS u32x4*>(stage + (isA ? 0 : Cfg::A_BYTES) + pos * 16) = v;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// MFMA over one stage
+// ---------------------------------------------------------------------------
+
+template <class Cfg, bool FIRST>
+__device__ inline void compute_stage(const IRIS_LDS char* stage, f32x16 (&acc)[Cfg::IM][Cfg::IN], int a_row_off,
+                                     int b_row_off, const int (&xoff)[Cfg::KSUB]) {
+  using V = typename Mfma<Cfg::DT>::vec8;
+  const IRIS_LDS char* sA = stage + a_row_off;
+  const IRIS_LDS char* sB = stage + Cfg::A_BYTES + b_row_off;
+  // all operand fragments of the K-step are requested up front; the MFMAs
+  // then start as the first ones arrive (LDS returns in order)
+  V a[Cfg::KSUB][Cfg::IM], b[Cfg::KSUB][Cfg::IN];
+#pragma unroll
+  for (int kk = 0; kk < Cfg::KSUB; ++kk) {
+#pragma unroll
+    for (int j = 0; j < Cfg::IN; ++j)
+      b[kk][j] = *reinterpret_cast<const IRIS_LDS V*>(sB + j * 32 * Cfg::BK * 2 + xoff[kk]);
+#pragma unroll
+    for (int i = 0; i < Cfg::IM; ++i)
+      a[kk][i] = *reinterpret_cast<const IRIS_LDS V*>(sA + i * 32 * Cfg::BK * 2 + xoff[kk]);
+  }
+  __builtin_amdgcn_sched_barrier(0);  // keep the fetches ahead of the MFMAs
+#pragma unroll
+  for (int kk = 0; kk < Cfg::KSUB; ++kk) {
+#pragma unroll
+    for (int i = 0; i < Cfg::IM; ++i)
+#pragma unroll
+      for (int j = 0; j < Cfg::IN; ++j) {
+        if (FIRST && kk == 0) {
+          const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          acc[i][j] = Mfma<Cfg::DT>::run(b[kk][j], a[kk][i], z);
+        } else {
+          acc[i][j] = Mfma<Cfg::DT>::run(b[kk][j], a[kk][i], acc[i][j]);
+        }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Epilogue
+// ---------------------------------------------------------------------------
+
+enum StoreOp { OP_STORE16 = 0, OP_STORE32 = 1, OP_ATOMIC32 = 2, OP_ATOMIC16 = 3 };
+
+// 16-bit atomic add on `p` (element type DT) by CAS on the containing word.
+template <int DT>
+__device__ inline void atomic_add16_cas(IRIS_GLOBAL unsigned short* p, float v) {
+  const uintptr_t addr = (uintptr_t)p;
+  IRIS_GLOBAL unsigned int* w = (IRIS_GLOBAL unsigned int*)(addr & ~(uintptr_t)3);
+  const int sh = (addr & 2) ? 16 : 0;
+  unsigned int old = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (;;) {
+    const unsigned short cur = (unsigned short)(old >> sh);
+    const unsigned short nv = to16<DT>(from16<DT>(cur) + v);
+    const unsigned int repl = (old & ~(0xFFFFu << sh)) | ((unsigned int)nv << sh);
+    if (__hip_atomic_compare_exchange_strong(w, &old, repl, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT))
+      break;
+  }
+}
+
+// Packed 2 x 16-bit atomic add on a 4-byte aligned pair.
+template <int DT>
+__device__ inline void atomic_add16_pair(IRIS_GLOBAL unsigned int* p, unsigned int v) {
+  if constexpr (DT == IRIS_DTYPE_BF16) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    __builtin_amdgcn_global_atomic_fadd_v2bf16((IRIS_GLOBAL bf16x2*)p,
+                                               __builtin_bit_cast(bf16x2, v));
+  } else {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    __builtin_amdgcn_global_atomic_fadd_v2f16((IRIS_GLOBAL f16x2*)p,
+                                              __builtin_bit_cast(f16x2, v));
+  }
+}
+
+// Write the wave's TM x TN accumulator block to `out` on the destination
+// ranks, rows < m_end, columns < n_end, through the wave-private LDS scratch.
+//
+// Accumulator layout (operands swapped): for block (i, j), register r, lane l:
+//   m = i*32 + l%32,   n = j*32 + 8*(r/4) + 4*(l/32) + r%4.
+//
+// A pass moves 32 rows x CP columns: registers -> scratch (16-byte units of a
+// row XOR-ed with the row index), then scratch -> memory with lanes running
+// along a row so that one instruction covers contiguous bytes.
+//
+// OP_STORE16 : 16-bit elements of type ODT        OP_STORE32 : fp32 elements
+// OP_ATOMIC32: fp32 atomic add                    OP_ATOMIC16: 16-bit atomic add
+template <class Cfg, int OP, int ODT>
+__device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM][Cfg::IN], IRIS_LDS char* ws,
+                                 int wm0, int wn0, int m_end, int n_end, int lane) {
+  constexpr bool F32 = (OP == OP_STORE32 || OP == OP_ATOMIC32);
+  constexpr int ES = F32 ? 4 : 2;
+  constexpr int CP = Cfg::WS_PITCH / ES;  // columns per pass
+  constexpr int NPASS = Cfg::TN / CP;     // 1 (16-bit) or 2 (fp32)
+  constexpr int NQ = CP / 8;              // 8-column groups per pass
+  constexpr int EPV = 16 / ES;            // elements per 16-byte unit
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  const int r_begin = p.dest_all ? 0 : p.cur_rank;
+  const int r_end = p.dest_all ? p.ws : p.cur_rank + 1;
+#pragma unroll
+  for (int i = 0; i < Cfg::IM; ++i) {
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      // ---- registers -> scratch
+      const int sw = (lrow / Cfg::ERPB) % Cfg::U16;
+#pragma unroll
+      for (int g = 0; g < NQ; ++g) {
+        const int gq = ps * NQ + g;  // 8-column group of the wave tile
+        const int j = gq / 4, q = gq % 4;
+        const float v0 = acc[i][j][q * 4 + 0], v1 = acc[i][j][q * 4 + 1];
+        const float v2 = acc[i][j][q * 4 + 2], v3 = acc[i][j][q * 4 + 3];
+        if constexpr (F32) {
+          const int u = (g * 2 + lhalf) ^ sw;
+          const f32x4 v = {v0, v1, v2, v3};
+          *reinterpret_cast<IRIS_LDS f32x4*>(ws + lrow * Cfg::WS_PITCH + u * 16) = v;
+        } else {
+          const int u = g ^ sw;
+          const u32x2 v = {pack2<ODT>(v0, v1), pack2<ODT>(v2, v3)};
+          *reinterpret_cast<IRIS_LDS u32x2*>(ws + lrow * Cfg::WS_PITCH + u * 16 + lhalf * 8) = v;
+        }
+      }
+      // ---- scratch -> memory
+      const int row0 = wm0 + i * 32, col0 = wn0 + ps * CP;
+      const bool interior = (row0 + 32 <= m_end) && (col0 + CP <= n_end);
+#pragma nounroll
+      for (int r = r_begin; r < r_end; ++r) {
+        IRIS_GLOBAL char* dst = rank_ptr(p, p.out, r);
+        if (OP == OP_ATOMIC32) {
+          // one fp32 per lane, lanes along the row
+          constexpr int ITER = 32 * CP / 64;
+#pragma unroll
+          for (int t = 0; t < ITER; ++t) {
+            const int idx = t * 64 + lane;
+            const int row = idx / CP, cc = idx % CP;
+            const int u = (cc / 4) ^ ((row / Cfg::ERPB) % Cfg::U16);
+            const float v =
+                *reinterpret_cast<const IRIS_LDS float*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 4) * 4);
+            const int m = row0 + row, n = col0 + cc;
+            if (m < m_end && n < n_end)
+              __hip_atomic_fetch_add((IRIS_GLOBAL float*)(dst + ((int64_t)m * p.som + (int64_t)n * p.son) * 4),
+                                     v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        } else if (interior && p.vec_out) {
+          if constexpr (OP == OP_ATOMIC16) {
+            // one packed pair per lane, lanes along the row
+            constexpr int ITER = 32 * (CP / 2) / 64;
+#pragma unroll
+            for (int t = 0; t < ITER; ++t) {
+              const int idx = t * 64 + lane;
+              const int row = idx / (CP / 2), cc = (idx % (CP / 2)) * 2;
+              const int u = (cc / 8) ^ ((row / Cfg::ERPB) % Cfg::U16);
+              const unsigned int v =
+                  *reinterpret_cast<const IRIS_LDS unsigned int*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 8) * 2);
+              const int m = row0 + row, n = col0 + cc;
+              atomic_add16_pair<ODT>((IRIS_GLOBAL unsigned int*)(dst + ((int64_t)m * p.som + n) * 2), v);
+            }
+          } else {
+            constexpr int RPI = 64 / Cfg::U16;  // rows per wave-wide 16-byte read
+#pragma unroll
+            for (int t = 0; t < 32 / RPI; ++t) {
+              const int row = t * RPI + lane / Cfg::U16;
+              const int u = lane % Cfg::U16;
+              const int pu = u ^ ((row / Cfg::ERPB) % Cfg::U16);
+              const u32x4 v = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + row * Cfg::WS_PITCH + pu * 16);
+              const int m = row0 + row, n = col0 + u * EPV;
+              *(IRIS_GLOBAL u32x4*)(dst + ((int64_t)m * p.som + n) * ES) = v;
+            }
+          }
+        } else {
+          // ragged edge or unaligned destination: element by element
+#pragma nounroll
+          for (int idx = lane; idx < 32 * CP; idx += 64) {
+            const int row = idx / CP, cc = idx % CP;
+            const int u = (cc / EPV) ^ ((row / Cfg::ERPB) % Cfg::U16);
+            const IRIS_LDS char* src = ws + row * Cfg::WS_PITCH + u * 16 + (cc % EPV) * ES;
+            const int m = row0 + row, n = col0 + cc;
+            if (m < m_end && n < n_end) {
+              IRIS_GLOBAL char* d = dst + ((int64_t)m * p.som + (int64_t)n * p.son) * ES;
+              if constexpr (OP == OP_STORE32)
+                *(IRIS_GLOBAL unsigned int*)d = *reinterpret_cast<const IRIS_LDS unsigned int*>(src);
+              else if constexpr (OP == OP_STORE16)
+                *(IRIS_GLOBAL unsigned short*)d = *reinterpret_cast<const IRIS_LDS unsigned short*>(src);
+              else
+                atomic_add16_cas<ODT>((IRIS_GLOBAL unsigned short*)d,
+                                      from16<ODT>(*reinterpret_cast<const IRIS_LDS unsigned short*>(src)));
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// Publish a finished logical tile: +1 (release) on the tile's flag of every
+// rank (flag_mode 1, the ready flag of the scatter epilogue) or of every
+// *other* rank (flag_mode 2, the ONE_SHOT producer signal,
+// gemm_one_shot_all_reduce.py:207-218).  One thread; the caller has made
+// every wave's stores complete and passed a barrier.
+__device__ inline void publish_tile(const GemmKArgs& p, int tile_id) {
+#pragma nounroll
+  for (int r = 0; r < p.ws; ++r) {
+    if (p.flag_mode == 2 && r == p.cur_rank) continue;
+    flag_add_release(rank_ptr(p, p.flags + tile_id, r), 1, p.sys != 0);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The kernel
+// ---------------------------------------------------------------------------
+
+template <class Cfg, int OP, int ODT>
+__global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  IRIS_LDS char* lds = (IRIS_LDS char*)lds_raw;
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int pid = xcd_remap(blockIdx.x, p.num_sms, p.num_xcds);
+
+  const int n_tiles = pid < p.total_tiles ? (p.total_tiles - pid + p.num_sms - 1) / p.num_sms : 0;
+  const int n_items = n_tiles * p.sub_m * p.sub_n;
+  const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
+  const int total_steps = n_items * nk;
+
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  IRIS_LDS char* ws = lds + Cfg::S * Cfg::STAGE + wave * Cfg::WS_BYTES;
+
+  // operand fetch offsets inside a stage
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  const int a_row_off = (wm * Cfg::TM + lrow) * Cfg::BK * 2;
+  const int b_row_off = (wn * Cfg::TN + lrow) * Cfg::BK * 2;
+  int xoff[Cfg::KSUB];
+#pragma unroll
+  for (int kk = 0; kk < Cfg::KSUB; ++kk) xoff[kk] = ((kk * 2 + lhalf) ^ ((lrow / Cfg::RP) % Cfg::CPR)) * 16;
+
+  f32x16 acc[Cfg::IM][Cfg::IN];
+#pragma unroll
+  for (int i = 0; i < Cfg::IM; ++i)
+#pragma unroll
+    for (int j = 0; j < Cfg::IN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // A tile's flag may only be published once every wave's stores of the tile
+  // have completed.  Waiting for that right after issuing them would stall
+  // the matrix cores, so the publication is deferred to the top of the next
+  // K-step, where the whole group waits on its memory counter anyway.
+  const bool defer_publish = Cfg::DMA && nk > 0 && p.flag_mode != 0;
+  int pending_tile = -1;
+
+  Loader<Cfg> ld;
+  int l_item = 0, l_k = 0;  // load cursor
+  Item l_it;
+  if (Cfg::DMA && total_steps > 0) {
+    l_it = decode_item<Cfg>(p, pid, 0);
+    ld.setup(p, l_it, wave, lane);
+#pragma unroll
+    for (int s = 0; s < Cfg::S - 1; ++s) {
+      if (s < total_steps) {
+        ld.issue(p, lds + s * Cfg::STAGE, l_k, wave);
+        if (++l_k == nk) {
+          l_k = 0;
+          ++l_item;
+          if (l_item < n_items) {
+            l_it = decode_item<Cfg>(p, pid, l_item);
+            ld.setup(p, l_it, wave, lane);
+          }
+        }
+      }
+    }
+  }
+
+  int c_item = 0, c_k = 0;  // compute cursor
+  Item c_it;
+  if (n_items > 0) c_it = decode_item<Cfg>(p, pid, 0);
+
+  // K == 0 leaves every tile all zeros: one epilogue per item, no loads.
+  const int n_outer = nk > 0 ? total_steps : n_items;
+  for (int g = 0; g < n_outer; ++g) {
+    if (nk > 0) {
+      IRIS_LDS char* stage = lds + (Cfg::DMA ? (g & (Cfg::S - 1)) : 0) * Cfg::STAGE;
+      if constexpr (Cfg::DMA) {
+        // wait for this step's slab; S-2 younger slabs may stay in flight
+        if (pending_tile >= 0 || g + Cfg::S - 2 > total_steps - 1 || Cfg::S < 3) {
+          IRIS_WAIT_VMCNT(0);
+        } else {
+          IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S > 2 ? Cfg::S - 2 : 0));
+        }
+        block_barrier_raw();  // slab visible to all waves; previous slab's readers done
+        if (pending_tile >= 0) {
+          if (tid == 0) publish_tile(p, pending_tile);
+          pending_tile = -1;
+        }
+        if (g + Cfg::S - 1 < total_steps) {
+          ld.issue(p, lds + ((g + Cfg::S - 1) & (Cfg::S - 1)) * Cfg::STAGE, l_k, wave);
+          if (++l_k == nk) {
+            l_k = 0;
+            ++l_item;
+            if (l_item < n_items) {
+              l_it = decode_item<Cfg>(p, pid, l_item);
+              ld.setup(p, l_it, wave, lane);
+            }
+          }
+        }
+      } else {
+        __syncthreads();  // previous step's readers are done with the stage
+        load_slab_generic<Cfg>(p, c_it, stage, c_k, tid);
+        __syncthreads();
+      }
+
+      if (c_k == 0) {
+        if (p.ts_begin && c_it.first_sub && tid == 0)
+          __hip_atomic_fetch_min((IRIS_GLOBAL unsigned long long*)(p.ts_begin + c_it.tile_id),
+                                 (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        compute_stage<Cfg, true>(stage, acc, a_row_off, b_row_off, xoff);
+      } else {
+        compute_stage<Cfg, false>(stage, acc, a_row_off, b_row_off, xoff);
+      }
+      if (++c_k < nk) continue;
+      c_k = 0;
+    }
+
+    // ---------------- epilogue of one compute tile ----------------
+    store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end, c_it.n_end,
+                            lane);
+    if (c_it.last_sub) {
+      if (defer_publish) {
+        pending_tile = c_it.tile_id;
+      } else if (p.flag_mode != 0) {
+        IRIS_WAIT_VMCNT(0);  // this wave's stores of the tile have completed
+        __syncthreads();
+        if (tid == 0) publish_tile(p, c_it.tile_id);
+      }
+      if (p.ts_end && tid == 0)
+        __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + c_it.tile_id),
+                               (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (++c_item < n_items) c_it = decode_item<Cfg>(p, pid, c_item);
+  }
+
+  if (pending_tile >= 0) {
+    IRIS_WAIT_VMCNT(0);
+    __syncthreads();
+    if (tid == 0) publish_tile(p, pending_tile);
+  }
+}
+
+}  // namespace iris_amd

@@ -1,0 +1,278 @@
+// C-ABI launcher of the persistent shard GEMM (include/iris_amd.h).
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+
+#include "gemm_registry.hpp"
+
+namespace iris_amd {
+
+namespace {
+
+const GemmKernelEntry* entries_for(int dt, int op, int* count) {
+  if (dt == IRIS_DTYPE_BF16) {
+    switch (op) {
+      case OP_STORE16: return gemm_entries_bf16_store16(count);
+      case OP_STORE32: return gemm_entries_bf16_store32(count);
+      case OP_ATOMIC32: return gemm_entries_bf16_atomic32(count);
+      case OP_ATOMIC16: return gemm_entries_bf16_atomic16(count);
+    }
+  } else if (dt == IRIS_DTYPE_F16) {
+    switch (op) {
+      case OP_STORE16: return gemm_entries_f16_store16(count);
+      case OP_STORE32: return gemm_entries_f16_store32(count);
+      case OP_ATOMIC32: return gemm_entries_f16_atomic32(count);
+      case OP_ATOMIC16: return gemm_entries_f16_atomic16(count);
+    }
+  }
+  *count = 0;
+  return nullptr;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// 16-byte vector access on a row-major [rows, cols] view of `es`-byte elements
+bool vec_ok(const void* base, int64_t stride_m, int64_t stride_n, int es) {
+  return stride_n == 1 && aligned16(base) && ((stride_m * es) % 16) == 0;
+}
+
+struct Plan {
+  const GemmKernelEntry* entry = nullptr;
+  GemmKArgs k{};
+  int fused_reduce = 0;  // ONE_SHOT with the CONSUME phase: follow with the reduce kernel
+};
+
+int dbg() {
+  static int v = std::getenv("IRIS_AMD_DEBUG") ? 1 : 0;
+  return v;
+}
+
+// Validate `a` and build the launch plan.  Returns hipSuccess,
+// hipErrorInvalidValue, or a pseudo-success with entry == nullptr when there
+// is no GEMM work to do.
+hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
+  if (a.M < 0 || a.N < 0 || a.K < 0) return hipErrorInvalidValue;
+  if (a.block_m <= 0 || a.block_n <= 0 || a.group_size_m <= 0) return hipErrorInvalidValue;
+  if (a.num_sms <= 0 || a.num_xcds <= 0 || (a.num_sms % a.num_xcds) != 0) return hipErrorInvalidValue;
+  if (a.world_size <= 0 || a.cur_rank < 0 || a.cur_rank >= a.world_size) return hipErrorInvalidValue;
+  if (a.world_size > 1 && a.heap_bases == nullptr) return hipErrorInvalidValue;
+  if (a.ab_dtype != IRIS_DTYPE_BF16 && a.ab_dtype != IRIS_DTYPE_F16) return hipErrorInvalidValue;
+
+  int op, out_dt;
+  GemmKArgs& k = plan->k;
+  k = GemmKArgs{};
+  switch (a.epilogue) {
+    case IRIS_EPI_ALL_SCATTER:
+      if (!a.c_global) return hipErrorInvalidValue;
+      out_dt = a.c_global_dtype;
+      op = out_dt == IRIS_DTYPE_F32 ? OP_STORE32 : OP_STORE16;
+      k.out = static_cast<char*>(a.c_global) +
+              (int64_t)a.cur_rank * a.N * a.stride_cn_global * dtype_size(out_dt);
+      k.som = a.stride_cm_global;
+      k.son = a.stride_cn_global;
+      k.dest_all = 1;
+      k.flag_mode = a.notify ? 1 : 0;
+      break;
+    case IRIS_EPI_ATOMIC_ADD:
+      if (!a.c_global) return hipErrorInvalidValue;
+      out_dt = a.c_global_dtype;
+      op = out_dt == IRIS_DTYPE_F32 ? OP_ATOMIC32 : OP_ATOMIC16;
+      k.out = static_cast<char*>(a.c_global);
+      k.som = a.stride_cm_global;
+      k.son = a.stride_cn_global;
+      k.dest_all = 1;
+      k.flag_mode = 0;
+      break;
+    case IRIS_EPI_ONE_SHOT:
+      if (!a.c || !a.c_global) return hipErrorInvalidValue;
+      if ((a.phase & ~IRIS_PHASE_FUSED) != 0 || a.phase == 0) return hipErrorInvalidValue;
+      out_dt = a.c_dtype;
+      op = out_dt == IRIS_DTYPE_F32 ? OP_STORE32 : OP_STORE16;
+      k.out = static_cast<char*>(a.c);
+      k.som = a.stride_cm;
+      k.son = a.stride_cn;
+      k.dest_all = 0;
+      k.flag_mode = 2;
+      plan->fused_reduce = (a.phase & IRIS_PHASE_CONSUME) ? 1 : 0;
+      if (!(a.phase & IRIS_PHASE_PRODUCE)) return hipSuccess;  // consumer only: no GEMM
+      break;
+    default:
+      return hipErrorInvalidValue;
+  }
+  if (out_dt != IRIS_DTYPE_F32 && out_dt != a.ab_dtype) return hipErrorInvalidValue;
+  if (k.flag_mode != 0 && a.world_size > 1 && !a.tile_completed) return hipErrorInvalidValue;
+  if (k.flag_mode == 1 && !a.tile_completed) return hipErrorInvalidValue;
+  if (a.M == 0 || a.N == 0) return hipSuccess;  // nothing to compute
+  if (!a.a || !a.b) {
+    if (a.K > 0) return hipErrorInvalidValue;
+  }
+
+  k.a = static_cast<const char*>(a.a);
+  k.b = static_cast<const char*>(a.b);
+  k.flags = a.tile_completed;
+  k.heap_bases = a.heap_bases;
+  k.ts_begin = a.mm_begin_timestamp;
+  k.ts_end = a.mm_end_timestamp;
+  k.sam = a.stride_am;
+  k.sak = a.stride_ak;
+  k.sbk = a.stride_bk;
+  k.sbn = a.stride_bn;
+  k.M = a.M;
+  k.N = a.N;
+  k.K = a.K;
+  k.BM = a.block_m;
+  k.BN = a.block_n;
+  k.G = a.group_size_m;
+  k.num_sms = a.num_sms;
+  k.num_xcds = a.num_xcds;
+  k.cur_rank = a.cur_rank;
+  k.ws = a.world_size;
+  k.num_pid_m = (a.M + a.block_m - 1) / a.block_m;
+  k.num_pid_n = (a.N + a.block_n - 1) / a.block_n;
+  k.total_tiles = k.num_pid_m * k.num_pid_n;
+  k.sys = a.scope == IRIS_SCOPE_SYSTEM;
+  k.vec_out = vec_ok(k.out, k.som, k.son, dtype_size(out_dt)) ? 1 : 0;
+
+  int count = 0;
+  const GemmKernelEntry* list = entries_for(a.ab_dtype, op, &count);
+  if (!list) return hipErrorInvalidValue;
+
+  // Operands fit the LDS-DMA loader when both are K-contiguous with 16-byte
+  // aligned rows and K is a multiple of 8; a compute tile's rows must stay
+  // within a 2 GiB window of its buffer descriptor.
+  const bool dma_ok = a.stride_ak == 1 && a.stride_bk == 1 && (a.stride_am % 8) == 0 && (a.stride_bn % 8) == 0 &&
+                      aligned16(a.a) && aligned16(a.b) && (a.K % 8) == 0 && a.stride_am > 0 && a.stride_bn > 0;
+  auto fits = [&](const GemmKernelEntry& e) {
+    if (!e.dma) return true;
+    if (!dma_ok) return false;
+    const int64_t lim = (int64_t)1 << 31;
+    return ((int64_t)e.cm * a.stride_am + a.K) * 2 < lim && ((int64_t)e.cn * a.stride_bn + a.K) * 2 < lim;
+  };
+
+  const GemmKernelEntry* pick = nullptr;
+  if (a.variant > 0) {
+    if (a.variant > count) return hipErrorInvalidValue;
+    const GemmKernelEntry& e = list[a.variant - 1];
+    if (!fits(e)) return hipErrorInvalidValue;
+    pick = &e;
+  } else {
+    // first entry whose compute tile divides the logical tile; the rows and
+    // columns a small matrix cannot fill are not worth a tall compute tile
+    for (int i = 0; i < count && !pick; ++i) {
+      const GemmKernelEntry& e = list[i];
+      if (!fits(e)) continue;
+      if (a.block_m % e.cm != 0 || a.block_n % e.cn != 0) continue;
+      if (e.cm > 64 && e.cm >= 2 * a.M) continue;
+      if (e.cn > 64 && e.cn >= 2 * a.N) continue;
+      pick = &e;
+    }
+    // otherwise the smallest tile that fits, with masked sub-tiles
+    for (int i = count - 1; i >= 0 && !pick; --i)
+      if (fits(list[i]) && list[i].cm == 64 && list[i].cn == 64) pick = &list[i];
+  }
+  if (!pick) return hipErrorInvalidValue;
+  // compute tiles per logical tile; a matrix smaller than one logical tile
+  // has nothing beyond its own edge
+  const int span_m = a.block_m < a.M ? a.block_m : a.M, span_n = a.block_n < a.N ? a.block_n : a.N;
+  k.sub_m = (span_m + pick->cm - 1) / pick->cm;
+  k.sub_n = (span_n + pick->cn - 1) / pick->cn;
+  plan->entry = pick;
+  return hipSuccess;
+}
+
+hipError_t ensure_lds(const GemmKernelEntry* e) {
+  // dynamic LDS above 64 KiB must be opted into once per function
+  static std::mutex m;
+  std::lock_guard<std::mutex> lock(m);
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             e->lds_bytes);
+}
+
+iris_reduce_args reduce_args_from(const iris_gemm_args& a) {
+  iris_reduce_args r{};
+  r.c = a.c;
+  r.c_global = a.c_global;
+  r.tile_completed = a.tile_completed;
+  r.heap_bases = a.heap_bases;
+  r.status = a.status;
+  r.M = a.M;
+  r.N = a.N;
+  r.stride_cm = a.stride_cm;
+  r.stride_cn = a.stride_cn;
+  r.stride_cm_global = a.stride_cm_global;
+  r.stride_cn_global = a.stride_cn_global;
+  r.block_m = a.block_m;
+  r.block_n = a.block_n;
+  r.group_size_m = a.group_size_m;
+  r.num_sms = a.num_sms;
+  r.num_xcds = a.num_xcds;
+  r.cur_rank = a.cur_rank;
+  r.world_size = a.world_size;
+  r.c_dtype = a.c_dtype;
+  r.c_global_dtype = a.c_global_dtype;
+  r.scope = a.scope;
+  r.wait_flags = 1;
+  r.variant = 0;
+  r.spin_timeout_ticks = a.spin_timeout_ticks;
+  return r;
+}
+
+}  // namespace
+}  // namespace iris_amd
+
+using namespace iris_amd;
+
+extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
+  if (!args) return hipErrorInvalidValue;
+  Plan plan;
+  hipError_t err = make_plan(*args, &plan);
+  if (err != hipSuccess) return err;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (plan.entry) {
+    const GemmKernelEntry* e = plan.entry;
+    if (e->lds_bytes > 64 * 1024) {
+      err = ensure_lds(e);
+      if (err != hipSuccess) return err;
+    }
+    if (dbg())
+      std::fprintf(stderr, "[iris_amd] gemm %s M=%d N=%d K=%d tiles=%d grid=%d sub=%dx%d lds=%d\n", e->name, plan.k.M,
+                   plan.k.N, plan.k.K, plan.k.total_tiles, plan.k.num_sms, plan.k.sub_m, plan.k.sub_n, e->lds_bytes);
+    hipLaunchKernelGGL(e->fn, dim3(plan.k.num_sms), dim3(e->threads), e->lds_bytes, s, plan.k);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+  }
+  if (plan.fused_reduce) {
+    // The consumer half of the one-shot epilogue runs as a second kernel on
+    // the same stream: it waits for each tile's flag, sums the partials and
+    // stores the result, exactly what the tail of the reference program does
+    // for that tile (gemm_one_shot_all_reduce.py:220-271).
+    const iris_reduce_args r = reduce_args_from(*args);
+    return iris_one_shot_reduce_launch(&r, stream);
+  }
+  return hipSuccess;
+}
+
+extern "C" int iris_gemm_kernel_info(const iris_gemm_args* args, int* n_regs, int* n_spills) {
+  if (!args) return hipErrorInvalidValue;
+  Plan plan;
+  hipError_t err = make_plan(*args, &plan);
+  if (err != hipSuccess) return err;
+  if (n_regs) *n_regs = 0;
+  if (n_spills) *n_spills = 0;
+  if (!plan.entry) return hipSuccess;
+  hipFuncAttributes attr;
+  err = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(plan.entry->fn));
+  if (err != hipSuccess) return err;
+  if (n_regs) *n_regs = attr.numRegs;
+  if (n_spills) *n_spills = static_cast<int>(attr.localSizeBytes);
+  return hipSuccess;
+}
+
+extern "C" int iris_gemm_variant_name(int ab_dtype, int out_is_f32, int atomic, int variant, char* buf, size_t len) {
+  const int op = atomic ? (out_is_f32 ? OP_ATOMIC32 : OP_ATOMIC16) : (out_is_f32 ? OP_STORE32 : OP_STORE16);
+  int count = 0;
+  const GemmKernelEntry* list = entries_for(ab_dtype, op, &count);
+  if (!list || variant < 1 || variant > count || !buf || len == 0) return hipErrorInvalidValue;
+  std::snprintf(buf, len, "%s", list[variant - 1].name);
+  return hipSuccess;
+}

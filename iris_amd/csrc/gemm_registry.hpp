@@ -1,0 +1,63 @@
+// Table of compiled shard-GEMM kernels.  Each instantiation file defines the
+// entries of one (operand type, epilogue op) pair; the launcher picks one
+// entry per call.
+#pragma once
+
+#include "gemm_kernel.hpp"
+
+namespace iris_amd {
+
+using GemmKernelFn = void (*)(const GemmKArgs);
+
+struct GemmKernelEntry {
+  int dt;      // operand type: IRIS_DTYPE_F16 | IRIS_DTYPE_BF16
+  int op;      // StoreOp
+  int cm, cn;  // compute tile
+  int bk, wm, wn, stages;
+  bool dma;    // LDS-DMA loader (needs K-contiguous, 16-byte aligned operands)
+  int threads;
+  int lds_bytes;
+  GemmKernelFn fn;
+  const char* name;
+};
+
+template <class Cfg, int OP>
+constexpr GemmKernelEntry make_entry(const char* name) {
+  constexpr int ODT = (OP == OP_STORE32 || OP == OP_ATOMIC32) ? IRIS_DTYPE_F32 : Cfg::DT;
+  return GemmKernelEntry{Cfg::DT, OP,      Cfg::CM, Cfg::CN, Cfg::BK,        Cfg::WM,
+                         Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::NT, Cfg::LDS_BYTES, &gemm_persistent_kernel<Cfg, OP, ODT>,
+                         name};
+}
+
+// The variants, in the launcher's order of preference: the first entry whose
+// compute tile divides the logical tile (and whose loader fits the operands)
+// wins.  `variant` k > 0 in iris_gemm_args forces entry k-1 (tuning runs).
+#define IRIS_GEMM_VARIANTS(X, DT, OP)                            \
+  X(DT, OP, 256, 256, 32, 2, 2, 4, true, "256x256x32_w2x2_s4")   \
+  X(DT, OP, 256, 128, 32, 2, 2, 4, true, "256x128x32_w2x2_s4")   \
+  X(DT, OP, 128, 256, 32, 2, 2, 4, true, "128x256x32_w2x2_s4")   \
+  X(DT, OP, 128, 128, 32, 2, 2, 4, true, "128x128x32_w2x2_s4")   \
+  X(DT, OP, 256, 64, 32, 4, 1, 4, true, "256x64x32_w4x1_s4")     \
+  X(DT, OP, 64, 64, 32, 2, 2, 4, true, "64x64x32_w2x2_s4")       \
+  X(DT, OP, 64, 64, 32, 2, 2, 1, false, "64x64x32_w2x2_generic")
+
+// extra variants of the headline tile, compiled for the bf16 store op only
+#define IRIS_GEMM_TUNING_VARIANTS(X, DT, OP)                     \
+  X(DT, OP, 256, 256, 32, 2, 4, 4, true, "256x256x32_w2x4_s4")   \
+  X(DT, OP, 256, 256, 64, 2, 2, 2, true, "256x256x64_w2x2_s2")   \
+  X(DT, OP, 256, 256, 64, 2, 4, 2, true, "256x256x64_w2x4_s2")
+
+#define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, NAME) \
+  make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP>(NAME),
+
+#define IRIS_GEMM_DECLARE(TAG) const GemmKernelEntry* gemm_entries_##TAG(int* count);
+IRIS_GEMM_DECLARE(bf16_store16)
+IRIS_GEMM_DECLARE(bf16_store32)
+IRIS_GEMM_DECLARE(bf16_atomic32)
+IRIS_GEMM_DECLARE(bf16_atomic16)
+IRIS_GEMM_DECLARE(f16_store16)
+IRIS_GEMM_DECLARE(f16_store32)
+IRIS_GEMM_DECLARE(f16_atomic32)
+IRIS_GEMM_DECLARE(f16_atomic16)
+
+}  // namespace iris_amd

@@ -1,0 +1,148 @@
+// C-ABI launchers of the one-shot reduce, the tile signal and the int32 fill
+// (include/iris_amd.h).
+#include <cstdio>
+#include <cstdlib>
+
+#include "reduce_kernel.hpp"
+
+namespace iris_amd {
+namespace {
+
+using ReduceFn = void (*)(const ReduceKArgs);
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <int IN_DT, int OUT_DT>
+ReduceFn pick_vec(int ws, int variant) {
+  // variant: 0 default; 1..6 tuning points of (UNROLL, nontemporal)
+  if (ws == 8) {
+    switch (variant) {
+      case 1: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 1, true>;
+      case 2: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 2, true>;
+      case 3: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 4, true>;
+      case 4: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 1, false>;
+      case 5: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 2, false>;
+      case 6: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 4, false>;
+      default: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 2, true>;
+    }
+  }
+  return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 0, 2, true>;
+}
+
+ReduceFn pick(int in_dt, int out_dt, int ws, int variant) {
+  if (in_dt == IRIS_DTYPE_F32) {
+    if (out_dt == IRIS_DTYPE_BF16) return pick_vec<IRIS_DTYPE_F32, IRIS_DTYPE_BF16>(ws, variant);
+    if (out_dt == IRIS_DTYPE_F16) return pick_vec<IRIS_DTYPE_F32, IRIS_DTYPE_F16>(ws, variant);
+    return pick_vec<IRIS_DTYPE_F32, IRIS_DTYPE_F32>(ws, variant);
+  }
+  if (in_dt == IRIS_DTYPE_BF16) {
+    if (out_dt == IRIS_DTYPE_BF16) return pick_vec<IRIS_DTYPE_BF16, IRIS_DTYPE_BF16>(ws, variant);
+    if (out_dt == IRIS_DTYPE_F32) return pick_vec<IRIS_DTYPE_BF16, IRIS_DTYPE_F32>(ws, variant);
+    return nullptr;
+  }
+  if (in_dt == IRIS_DTYPE_F16) {
+    if (out_dt == IRIS_DTYPE_F16) return pick_vec<IRIS_DTYPE_F16, IRIS_DTYPE_F16>(ws, variant);
+    if (out_dt == IRIS_DTYPE_F32) return pick_vec<IRIS_DTYPE_F16, IRIS_DTYPE_F32>(ws, variant);
+    return nullptr;
+  }
+  return nullptr;
+}
+
+bool valid_dtype(int dt) { return dt == IRIS_DTYPE_F32 || dt == IRIS_DTYPE_F16 || dt == IRIS_DTYPE_BF16; }
+
+}  // namespace
+}  // namespace iris_amd
+
+using namespace iris_amd;
+
+extern "C" int iris_one_shot_reduce_launch(const iris_reduce_args* a, void* stream) {
+  if (!a) return hipErrorInvalidValue;
+  if (a->M < 0 || a->N < 0 || a->block_m <= 0 || a->block_n <= 0 || a->group_size_m <= 0) return hipErrorInvalidValue;
+  if (a->world_size <= 0 || a->cur_rank < 0 || a->cur_rank >= a->world_size) return hipErrorInvalidValue;
+  if (a->world_size > 1 && !a->heap_bases) return hipErrorInvalidValue;
+  if (a->wait_flags && a->world_size > 1 && !a->tile_completed) return hipErrorInvalidValue;
+  if (!valid_dtype(a->c_dtype) || !valid_dtype(a->c_global_dtype)) return hipErrorInvalidValue;
+  if (a->num_sms < 0 || a->num_xcds <= 0) return hipErrorInvalidValue;
+  if (a->M == 0 || a->N == 0) return hipSuccess;
+  if (!a->c || !a->c_global) return hipErrorInvalidValue;
+
+  ReduceKArgs k{};
+  k.c = static_cast<const char*>(a->c);
+  k.cg = static_cast<char*>(a->c_global);
+  k.flags = a->tile_completed;
+  k.heap_bases = a->heap_bases;
+  k.status = a->status;
+  k.timeout = a->spin_timeout_ticks ? a->spin_timeout_ticks : 200000000ull;  // 2 s at 100 MHz
+  k.scm = a->stride_cm;
+  k.scn = a->stride_cn;
+  k.sgm = a->stride_cm_global;
+  k.sgn = a->stride_cn_global;
+  k.M = a->M;
+  k.N = a->N;
+  k.BM = a->block_m;
+  k.BN = a->block_n;
+  k.G = a->group_size_m;
+  k.num_pid_m = (a->M + a->block_m - 1) / a->block_m;
+  k.num_pid_n = (a->N + a->block_n - 1) / a->block_n;
+  k.total_tiles = k.num_pid_m * k.num_pid_n;
+  k.cur_rank = a->cur_rank;
+  k.ws = a->world_size;
+  k.c_dt = a->c_dtype;
+  k.cg_dt = a->c_global_dtype;
+  k.sys = a->scope == IRIS_SCOPE_SYSTEM;
+  k.wait_flags = a->wait_flags;
+
+  int grid = a->num_sms > 0 ? a->num_sms : k.total_tiles;
+  if (grid > k.total_tiles) grid = k.total_tiles;
+  // the XCD remap is a permutation only when the grid splits evenly
+  k.num_xcds = (a->num_xcds > 1 && grid % a->num_xcds == 0) ? a->num_xcds : 1;
+
+  const int ies = dtype_size(k.c_dt), oes = dtype_size(k.cg_dt);
+  const bool vec = k.scn == 1 && k.sgn == 1 && aligned16(k.c) && aligned16(k.cg) && (k.scm * ies) % 16 == 0 &&
+                   (k.sgm * oes) % 16 == 0 && k.BN % 8 == 0 && k.N % 8 == 0;
+  ReduceFn fn = vec ? pick(k.c_dt, k.cg_dt, k.ws, a->variant) : nullptr;
+  if (!fn) fn = &reduce_tiles_generic_kernel;
+  hipLaunchKernelGGL(fn, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), k);
+  return hipGetLastError();
+}
+
+extern "C" int iris_signal_tiles_launch(int32_t* tile_completed, const uint64_t* heap_bases, int32_t total_tiles,
+                                        int32_t cur_rank, int32_t world_size, int32_t include_self, int32_t scope,
+                                        void* stream) {
+  if (total_tiles < 0 || world_size <= 0 || cur_rank < 0 || cur_rank >= world_size) return hipErrorInvalidValue;
+  if (total_tiles == 0) return hipSuccess;
+  if (!tile_completed || (world_size > 1 && !heap_bases)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(signal_tiles_kernel, dim3((total_tiles + 255) / 256), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), tile_completed, heap_bases, total_tiles, cur_rank, world_size,
+                     include_self, scope == IRIS_SCOPE_SYSTEM ? 1 : 0);
+  return hipGetLastError();
+}
+
+extern "C" int iris_memset_i32_launch(int32_t* ptr, int32_t value, int64_t n_elements, void* stream) {
+  if (n_elements < 0) return hipErrorInvalidValue;
+  if (n_elements == 0) return hipSuccess;
+  if (!ptr) return hipErrorInvalidValue;
+  const int64_t blocks = (n_elements + 1023) / 1024;
+  hipLaunchKernelGGL(memset_i32_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), ptr,
+                     value, n_elements);
+  return hipGetLastError();
+}
+
+extern "C" int iris_tile_schedule_launch(int32_t* out, int32_t M, int32_t N, int32_t block_m, int32_t block_n,
+                                         int32_t group_size_m, int32_t num_sms, int32_t num_xcds, void* stream) {
+  if (M <= 0 || N <= 0 || block_m <= 0 || block_n <= 0 || group_size_m <= 0 || num_sms <= 0 || num_xcds <= 0 ||
+      num_sms % num_xcds != 0 || !out)
+    return hipErrorInvalidValue;
+  const int npm = (M + block_m - 1) / block_m, npn = (N + block_n - 1) / block_n;
+  hipLaunchKernelGGL(tile_schedule_kernel, dim3((num_sms + 255) / 256), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), out, npm, npn, group_size_m, num_sms, num_xcds);
+  return hipGetLastError();
+}
+
+extern "C" void iris_tile_map_host(int32_t tile_id, int32_t M, int32_t N, int32_t block_m, int32_t block_n,
+                                   int32_t group_size_m, int32_t* pid_m, int32_t* pid_n) {
+  const TileCoord tc =
+      tile_map(tile_id, (M + block_m - 1) / block_m, (N + block_n - 1) / block_n, group_size_m);
+  *pid_m = tc.pid_m;
+  *pid_n = tc.pid_n;
+}

@@ -1,0 +1,309 @@
+"""Python launchers of the HIP kernels, over the C-ABI of ``libiris_amd.so``.
+
+These check operand shapes against what the kernels and their grids assume
+*before* anything is launched, fill the C argument structs and launch on
+torch's current stream.  They never synchronise and never allocate.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _native
+from ._native import (
+    DTYPE_BF16,
+    DTYPE_F16,
+    DTYPE_F32,
+    EPI_ALL_SCATTER,
+    EPI_ATOMIC_ADD,
+    EPI_ONE_SHOT,
+    PHASE_CONSUME,
+    PHASE_FUSED,
+    PHASE_PRODUCE,
+    SCOPE_AGENT,
+    SCOPE_SYSTEM,
+)
+
+__all__ = [
+    "gemm_launch",
+    "gemm_kernel_info",
+    "gemm_variant_name",
+    "one_shot_reduce",
+    "signal_tiles",
+    "tile_schedule",
+    "tile_map_host",
+    "cdiv",
+    "default_num_xcds",
+    "EPI_ALL_SCATTER",
+    "EPI_ATOMIC_ADD",
+    "EPI_ONE_SHOT",
+    "PHASE_PRODUCE",
+    "PHASE_CONSUME",
+    "PHASE_FUSED",
+    "SCOPE_AGENT",
+    "SCOPE_SYSTEM",
+]
+
+_DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
+
+
+def cdiv(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def default_num_xcds(cu_count: int, num_sms: int) -> int:
+    """XCDs to spread the persistent programs over.
+
+    The reference hard-codes "8 iff 304 CUs" (matmul_wrapper.py:63-65, the
+    MI300X).  An MI355X has 8 XCDs of 32 CUs; workgroups are dealt to XCDs
+    round-robin, so the same remap keeps neighbouring tiles on one XCD's L2.
+    The remap only changes which CU computes a tile, never a result or flag.
+    """
+    if cu_count in (304, 256) and num_sms % 8 == 0:
+        return 8
+    return 1
+
+
+def _dtype_code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f"{what}: unsupported dtype {t.dtype}") from None
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _require_cuda(what: str, t: torch.Tensor, device: torch.device):
+    if not t.is_cuda or t.device != device:
+        raise RuntimeError(f"{what} must be on {device}, got {t.device}")
+
+
+def _extent_ok(t: torch.Tensor, rows: int, cols: int) -> bool:
+    return t.dim() == 2 and t.shape[0] >= rows and t.shape[1] >= cols
+
+
+def _check_flags(tile_completed, total_tiles, device):
+    if tile_completed is None:
+        return
+    _require_cuda("tile_completed", tile_completed, device)
+    if tile_completed.dtype != torch.int32 or not tile_completed.is_contiguous():
+        raise TypeError("tile_completed must be a contiguous int32 tensor")
+    if tile_completed.numel() < total_tiles:
+        raise ValueError(f"tile_completed has {tile_completed.numel()} flags, {total_tiles} tiles need one each")
+
+
+def _check_heap_bases(heap_bases, world_size, device):
+    if heap_bases is None:
+        if world_size > 1:
+            raise ValueError("heap_bases is required when world_size > 1")
+        return
+    _require_cuda("heap_bases", heap_bases, device)
+    if heap_bases.dtype not in (torch.uint64, torch.int64) or heap_bases.numel() < world_size:
+        raise TypeError("heap_bases must hold one 64-bit base address per rank")
+
+
+def _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
+                    gsize_m, epilogue, phase, notify, num_xcds, scope, variant, mm_begin_timestamp,
+                    mm_end_timestamp, status, spin_timeout_ticks):
+    assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0], "incompatible dimensions"
+    device = a.device
+    M, K = a.shape
+    _, N = b.shape
+    _require_cuda("a", a, device)
+    _require_cuda("b", b, device)
+    if a.dtype != b.dtype:
+        raise TypeError(f"a and b must share a dtype, got {a.dtype} and {b.dtype}")
+    if a.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError(f"operands must be fp16 or bf16, got {a.dtype}")
+    if BLK_M <= 0 or BLK_N <= 0 or gsize_m <= 0 or num_sms <= 0:
+        raise ValueError("block sizes, gsize_m and the grid must be positive")
+    total_tiles = cdiv(M, BLK_M) * cdiv(N, BLK_N)
+
+    if epilogue == EPI_ALL_SCATTER:
+        # rank r's columns land at offset r*N of c_global[M, N*world_size]
+        if c_global is None or not _extent_ok(c_global, M, N * world_size):
+            raise ValueError(f"c_global must be at least [{M}, {N * world_size}] for the all-scatter epilogue")
+    elif epilogue == EPI_ATOMIC_ADD:
+        if c_global is None or not _extent_ok(c_global, M, N):
+            raise ValueError(f"c_global must be at least [{M}, {N}]")
+    elif epilogue == EPI_ONE_SHOT:
+        if c is None or not _extent_ok(c, M, N):
+            raise ValueError(f"c must be at least [{M}, {N}]")
+        if c_global is None or not _extent_ok(c_global, M, N):
+            raise ValueError(f"c_global must be at least [{M}, {N}]")
+    else:
+        raise ValueError(f"unknown epilogue {epilogue}")
+    for name, t in (("c", c), ("c_global", c_global)):
+        if t is not None:
+            _require_cuda(name, t, device)
+    _check_flags(tile_completed, total_tiles, device)
+    _check_heap_bases(heap_bases, world_size, device)
+    for name, t in (("mm_begin_timestamp", mm_begin_timestamp), ("mm_end_timestamp", mm_end_timestamp)):
+        if t is not None:
+            _require_cuda(name, t, device)
+            if t.dtype != torch.int64 or t.numel() < total_tiles or not t.is_contiguous():
+                raise TypeError(f"{name} must be a contiguous int64 tensor with one entry per tile")
+    if status is not None:
+        _require_cuda("status", status, device)
+        if status.dtype not in (torch.int32, torch.uint32) or status.numel() < 1:
+            raise TypeError("status must be a 32-bit device word")
+
+    args = _native.GemmArgs()
+    args.a, args.b = _ptr(a), _ptr(b)
+    args.c, args.c_global = _ptr(c), _ptr(c_global)
+    args.tile_completed = _ptr(tile_completed)
+    args.heap_bases = _ptr(heap_bases)
+    args.mm_begin_timestamp = _ptr(mm_begin_timestamp)
+    args.mm_end_timestamp = _ptr(mm_end_timestamp)
+    args.status = _ptr(status)
+    args.M, args.N, args.K = M, N, K
+    args.stride_am, args.stride_ak = a.stride(0), a.stride(1)
+    args.stride_bk, args.stride_bn = b.stride(0), b.stride(1)
+    if c is not None:
+        args.stride_cm, args.stride_cn = c.stride(0), c.stride(1)
+        args.c_dtype = _dtype_code(c, "c")
+    if c_global is not None:
+        args.stride_cm_global, args.stride_cn_global = c_global.stride(0), c_global.stride(1)
+        args.c_global_dtype = _dtype_code(c_global, "c_global")
+    args.block_m, args.block_n, args.block_k = BLK_M, BLK_N, BLK_K
+    args.group_size_m = gsize_m
+    args.num_sms = num_sms
+    args.num_xcds = num_xcds
+    args.cur_rank, args.world_size = rank, world_size
+    args.ab_dtype = _dtype_code(a, "a")
+    args.epilogue = epilogue
+    args.phase = phase
+    args.notify = 1 if notify else 0
+    args.scope = scope
+    args.variant = variant
+    args.spin_timeout_ticks = spin_timeout_ticks
+    return args
+
+
+def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
+                gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, scope=SCOPE_AGENT, variant=0,
+                mm_begin_timestamp=None, mm_end_timestamp=None, status=None, spin_timeout_ticks=0):
+    """Launch the persistent shard GEMM ``a @ b`` with a tile-publishing epilogue.
+
+    The kernel launch of the reference wrappers (matmul_wrapper.py:109-150).
+    """
+    args = _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N,
+                           BLK_K, gsize_m, epilogue, phase, notify, num_xcds, scope, variant, mm_begin_timestamp,
+                           mm_end_timestamp, status, spin_timeout_ticks)
+    stream = torch.cuda.current_stream(a.device).cuda_stream
+    with torch.cuda.device(a.device):
+        err = _native.lib().iris_gemm_launch(ctypes.byref(args), stream)
+    if err == _native.HIP_ERROR_INVALID_VALUE:
+        raise ValueError(
+            "iris_gemm_launch rejected the arguments (shape, strides, dtypes, grid or rank layout it does not take)"
+        )
+    _native.hip_try(err)
+
+
+def gemm_kernel_info(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
+                     gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, variant=0):
+    """(registers, spill bytes per lane) of the kernel a launch would use."""
+    args = _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N,
+                           BLK_K, gsize_m, epilogue, phase, notify, num_xcds, SCOPE_AGENT, variant, None, None, None,
+                           0)
+    regs, spills = ctypes.c_int(), ctypes.c_int()
+    with torch.cuda.device(a.device):
+        _native.hip_try(_native.lib().iris_gemm_kernel_info(ctypes.byref(args), ctypes.byref(regs),
+                                                            ctypes.byref(spills)))
+    return regs.value, spills.value
+
+
+def gemm_variant_name(dtype: torch.dtype, out_is_f32: bool, atomic: bool, variant: int) -> Optional[str]:
+    buf = ctypes.create_string_buffer(128)
+    err = _native.lib().iris_gemm_variant_name(_DTYPES[dtype], int(out_is_f32), int(atomic), variant, buf, 128)
+    return None if err else buf.value.decode()
+
+
+def one_shot_reduce(c, c_global, tile_completed, heap_bases, rank, world_size, BLK_M, BLK_N, gsize_m, *,
+                    num_sms=0, num_xcds=1, scope=SCOPE_AGENT, wait_flags=True, variant=0, status=None,
+                    spin_timeout_ticks=0):
+    """Sum the ``world_size`` partial buffers that sit at ``c``'s heap offset on
+    every rank into ``c_global``, tile by tile, behind the tiles' flags.
+
+    The consumer half of gemm_one_shot_all_reduce.py:220-271.
+    """
+    if c.dim() != 2 or c_global.dim() != 2:
+        raise ValueError("c and c_global must be matrices")
+    M, N = c.shape
+    device = c.device
+    _require_cuda("c", c, device)
+    _require_cuda("c_global", c_global, device)
+    if not _extent_ok(c_global, M, N):
+        raise ValueError(f"c_global must be at least [{M}, {N}]")
+    if BLK_M <= 0 or BLK_N <= 0 or gsize_m <= 0 or num_sms < 0:
+        raise ValueError("block sizes and gsize_m must be positive")
+    total_tiles = cdiv(M, BLK_M) * cdiv(N, BLK_N)
+    if wait_flags and world_size > 1 and tile_completed is None:
+        raise ValueError("tile_completed is required to wait on flags")
+    _check_flags(tile_completed, total_tiles, device)
+    _check_heap_bases(heap_bases, world_size, device)
+    args = _native.ReduceArgs()
+    args.c, args.c_global = _ptr(c), _ptr(c_global)
+    args.tile_completed = _ptr(tile_completed)
+    args.heap_bases = _ptr(heap_bases)
+    args.status = _ptr(status)
+    args.M, args.N = M, N
+    args.stride_cm, args.stride_cn = c.stride(0), c.stride(1)
+    args.stride_cm_global, args.stride_cn_global = c_global.stride(0), c_global.stride(1)
+    args.block_m, args.block_n, args.group_size_m = BLK_M, BLK_N, gsize_m
+    args.num_sms, args.num_xcds = num_sms, num_xcds
+    args.cur_rank, args.world_size = rank, world_size
+    args.c_dtype, args.c_global_dtype = _dtype_code(c, "c"), _dtype_code(c_global, "c_global")
+    args.scope = scope
+    args.wait_flags = 1 if wait_flags else 0
+    args.variant = variant
+    args.spin_timeout_ticks = spin_timeout_ticks
+    stream = torch.cuda.current_stream(device).cuda_stream
+    with torch.cuda.device(device):
+        err = _native.lib().iris_one_shot_reduce_launch(ctypes.byref(args), stream)
+    if err == _native.HIP_ERROR_INVALID_VALUE:
+        raise ValueError("iris_one_shot_reduce_launch rejected the arguments")
+    _native.hip_try(err)
+
+
+def tile_schedule(M, N, BLK_M, BLK_N, gsize_m, num_sms, num_xcds, device="cuda"):
+    """int32[total_tiles, 4] = (pid_m, pid_n, program, position) per tile id,
+    computed on the device by the functions the kernels use."""
+    total = cdiv(M, BLK_M) * cdiv(N, BLK_N)
+    out = torch.full((total, 4), -1, dtype=torch.int32, device=device)
+    stream = torch.cuda.current_stream(out.device).cuda_stream
+    with torch.cuda.device(out.device):
+        err = _native.lib().iris_tile_schedule_launch(out.data_ptr(), M, N, BLK_M, BLK_N, gsize_m, num_sms,
+                                                      num_xcds, stream)
+    if err == _native.HIP_ERROR_INVALID_VALUE:
+        raise ValueError("iris_tile_schedule_launch rejected the arguments")
+    _native.hip_try(err)
+    return out
+
+
+def tile_map_host(tile_id, M, N, BLK_M, BLK_N, gsize_m):
+    """(pid_m, pid_n) from the host build of the kernels' tile map."""
+    pm, pn = ctypes.c_int32(), ctypes.c_int32()
+    _native.lib().iris_tile_map_host(tile_id, M, N, BLK_M, BLK_N, gsize_m, ctypes.byref(pm), ctypes.byref(pn))
+    return pm.value, pn.value
+
+
+def signal_tiles(tile_completed, heap_bases, total_tiles, rank, world_size, *, include_self=False,
+                 scope=SCOPE_AGENT):
+    """+1 (release) on the flag of every tile on the other ranks (on every rank
+    with ``include_self``); gemm_one_shot_all_reduce.py:207-218 on its own."""
+    device = tile_completed.device
+    _check_flags(tile_completed, total_tiles, device)
+    _check_heap_bases(heap_bases, world_size, device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    with torch.cuda.device(device):
+        err = _native.lib().iris_signal_tiles_launch(tile_completed.data_ptr(), _ptr(heap_bases), total_tiles, rank,
+                                                     world_size, 1 if include_self else 0, scope, stream)
+    if err == _native.HIP_ERROR_INVALID_VALUE:
+        raise ValueError("iris_signal_tiles_launch rejected the arguments")
+    _native.hip_try(err)

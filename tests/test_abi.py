@@ -1,0 +1,110 @@
+"""The C-ABI: both libraries load and export every symbol ``include/iris_amd.h``
+declares, and the ctypes structs have the layout the C compiler gives them.
+No compute call is made."""
+
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+from iris_amd import _native
+
+ROOT = os.path.abspath(os.path.join(os.path.dirname(__file__), ".."))
+HEADER = os.path.join(ROOT, "include", "iris_amd.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(iris_[a-z0-9_]+|finegrained_hip[A-Za-z]+)\s*\(", text)))
+
+
+def test_header_and_bindings_name_the_same_functions():
+    names = declared_functions()
+    lib_names = [n for n in names if n.startswith("iris_")]
+    assert sorted(lib_names) == sorted(_native.SIGNATURES)
+    assert sorted(n for n in names if n.startswith("finegrained_")) == sorted(_native.ALLOCATOR_SYMBOLS)
+
+
+def test_libraries_load_and_export_every_declared_symbol():
+    lib = _native.lib()
+    for name in _native.SIGNATURES:
+        assert getattr(lib, name) is not None
+    assert lib.iris_amd_abi_version() == 1
+    alloc = ctypes.CDLL(_native.ALLOCATOR_LIB_PATH)
+    for name in _native.ALLOCATOR_SYMBOLS:
+        assert getattr(alloc, name) is not None
+
+
+def test_struct_layout_matches_the_c_compiler(tmp_path):
+    def probe(struct, cname):
+        lines = [f'printf("%zu\\n", sizeof({cname}));']
+        for fname, _ in struct._fields_:
+            lines.append(f'printf("{fname} %zu\\n", offsetof({cname}, {fname}));')
+        return "\n".join(lines)
+
+    src = tmp_path / "layout.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "iris_amd.h"\nint main(void){\n'
+        + probe(_native.GemmArgs, "iris_gemm_args") + 'printf("--\\n");' + probe(_native.ReduceArgs, "iris_reduce_args")
+        + "return 0;}\n"
+    )
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o",
+                    str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    first, second = out.split("--\n")
+    for struct, block in ((_native.GemmArgs, first), (_native.ReduceArgs, second)):
+        rows = block.strip().splitlines()
+        assert int(rows[0]) == ctypes.sizeof(struct)
+        for row in rows[1:]:
+            name, off = row.split()
+            assert getattr(struct, name).offset == int(off), name
+
+
+def test_error_strings_and_missing_library_is_loud(monkeypatch):
+    assert b"invalid" in _native.lib().iris_hip_error_string(1).lower()
+    with pytest.raises(RuntimeError, match="HIP error code 1"):
+        _native.hip_try(1)
+    _native.hip_try(0)
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "LIB_PATH", "/nonexistent/libiris_amd.so")
+    with pytest.raises(RuntimeError, match="no other implementation"):
+        _native.lib()
+
+
+def test_launchers_reject_bad_arguments_without_a_device():
+    lib = _native.lib()
+    assert lib.iris_gemm_launch(None, None) == _native.HIP_ERROR_INVALID_VALUE
+    g = _native.GemmArgs()  # all zero: no block sizes, no grid
+    assert lib.iris_gemm_launch(ctypes.byref(g), None) == _native.HIP_ERROR_INVALID_VALUE
+    g.block_m = g.block_n = g.group_size_m = g.num_sms = g.num_xcds = g.world_size = 1
+    g.ab_dtype = _native.DTYPE_F32  # operands must be 16-bit
+    assert lib.iris_gemm_launch(ctypes.byref(g), None) == _native.HIP_ERROR_INVALID_VALUE
+    g.ab_dtype = _native.DTYPE_BF16
+    g.num_sms, g.num_xcds = 12, 8  # the XCD remap needs an even split
+    assert lib.iris_gemm_launch(ctypes.byref(g), None) == _native.HIP_ERROR_INVALID_VALUE
+    r = _native.ReduceArgs()
+    assert lib.iris_one_shot_reduce_launch(ctypes.byref(r), None) == _native.HIP_ERROR_INVALID_VALUE
+    assert lib.iris_signal_tiles_launch(None, None, 4, 0, 0, 0, 0, None) == _native.HIP_ERROR_INVALID_VALUE
+    assert lib.iris_memset_i32_launch(None, 0, -1, None) == _native.HIP_ERROR_INVALID_VALUE
+    assert lib.iris_memset_i32_launch(None, 0, 0, None) == 0  # empty fill is a no-op
+
+
+def test_host_build_of_the_kernel_tile_map_is_bit_exact():
+    """The kernels' tile_map function, compiled for the host, against the
+    oracle over whole tile grids (the same source is compiled for the
+    device; the GPU tests check that build)."""
+    from iris_amd import ops
+    from oracle import iris_oracle as O
+
+    for M, N, BM, BN, G in [(8192, 8192, 256, 256, 4), (8192, 8192, 256, 256, 6), (4096, 4096, 256, 256, 6),
+                            (2048, 1376, 256, 64, 4), (1, 1376, 256, 256, 8), (1000, 999, 64, 64, 5),
+                            (8192, 4608, 256, 64, 4), (768, 512, 256, 128, 6)]:
+        total = O.cdiv(M, BM) * O.cdiv(N, BN)
+        want = O.tile_map_all(M, N, BM, BN, G)
+        got = [ops.tile_map_host(t, M, N, BM, BN, G) for t in range(total)]
+        assert got == [tuple(r) for r in want.tolist()]

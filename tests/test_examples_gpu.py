@@ -1,0 +1,43 @@
+"""The three example drivers end to end (CLI -> matmul.apply -> HIP kernel ->
+validate_gemm), at small sizes."""
+
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.abspath(os.path.join(os.path.dirname(__file__), ".."))
+
+
+def run_example(tmp_path, example, *argv):
+    out = tmp_path / "log.json"
+    cmd = [sys.executable, "-u", os.path.join(ROOT, "examples", example, "benchmark.py"), "--output_file", str(out),
+           "--heap_size", str(1 << 28), *argv]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300, cwd=str(tmp_path))
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    return json.loads(out.read_text()), proc.stdout
+
+
+@pytest.mark.parametrize("example,extra", [
+    ("07_gemm_all_scatter", ["--BLK_M", "256", "--BLK_N", "64"]),
+    ("08_gemm_atomics_all_reduce", ["--BLK_M", "256", "--BLK_N", "128"]),
+    ("09_gemm_one_shot_all_reduce", ["--BLK_M", "256", "--BLK_N", "256"]),
+])
+def test_example_validates(tmp_path, example, extra):
+    data, stdout = run_example(tmp_path, example, "-m", "1024", "-n", "768", "-k", "512", "--datatype", "bf16", "-v",
+                               "-d", *extra)
+    assert data["success"] is True
+    assert data["world_size"] == 1 and data["gemm_sms"] == 256
+    assert data["gemm_registers"] > 0 and data["gemm_spills"] == 0
+    assert "Final C validation passed." in stdout and "registers used" in stdout
+
+
+def test_one_shot_example_with_virtual_ranks_and_benchmark(tmp_path):
+    data, _ = run_example(tmp_path, "09_gemm_one_shot_all_reduce", "-m", "512", "-n", "512", "-k", "1024",
+                          "--datatype", "fp16", "-v", "-b", "--virtual_ranks", "4", "--BLK_N", "128")
+    assert data["success"] is True and data["world_size"] == 4 and data["k"] == 256
+    assert data["triton_ms"] > 0 and data["triton_tflops"] > 0 and data["gemm_experiments"] == 126

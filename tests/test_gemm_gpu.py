@@ -1,0 +1,398 @@
+"""Parity of the HIP shard GEMM and its three epilogues against the CPU
+oracle, through the C-ABI (``iris_amd.ops`` -> ``libiris_amd.so``).
+
+Values: rtol 1e-2 / atol 1e-2 against the fp32-accumulated oracle (the K-block
+order inside the matrix cores is not pinned by the reference).  Flags and
+tile indices: bit-exact.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from iris_amd import ops
+from oracle import iris_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-2, 1e-2
+
+
+def make_ab(M, N, K, dtype, scale=0.02, seed=123, lda=None, ldb=None):
+    """Seeded A [M,K] row-major and B [K,N] K-contiguous (the reference's TN
+    layout, benchmark.py:101-102); optional leading dimensions > K give the
+    strided K-shard views of 08/09."""
+    g = torch.Generator().manual_seed(seed)
+    lda, ldb = lda or K, ldb or K
+    Af = (torch.randn(M, lda, generator=g) * scale).to(dtype)
+    Bf = (torch.randn(N, ldb, generator=g) * scale).to(dtype)
+    return Af[:, :K], Bf[:, :K].T
+
+
+def to_heap(shmem, t):
+    """Copy a (possibly strided) host matrix into the heap, keeping its strides."""
+    rows, cols = t.shape
+    if t.stride(1) == 1:  # row-major view with leading dimension stride(0)
+        buf = shmem.zeros((rows, t.stride(0)), dtype=t.dtype)
+        buf[:, :cols].copy_(t)
+        return buf[:, :cols]
+    assert t.stride(0) == 1  # column-major view (B): store the transpose
+    buf = shmem.zeros((cols, t.stride(1)), dtype=t.dtype)
+    buf[:, :rows].copy_(t.T)
+    return buf[:, :rows].T
+
+
+def check_close(got, want, what=""):
+    got, want = got.float().cpu(), want.float().cpu()
+    bad = ~torch.isclose(got, want, rtol=RTOL, atol=ATOL)
+    assert not bad.any(), f"{what}: {int(bad.sum())} mismatches, max abs err {(got - want).abs().max().item()}"
+
+
+SCATTER_CASES = [
+    # M, N, K, BLK_M, BLK_N, G, grid, dtype
+    (256, 256, 64, 256, 256, 4, 4, torch.bfloat16),
+    (512, 768, 256, 256, 256, 4, 256, torch.bfloat16),
+    (512, 768, 256, 256, 256, 6, 8, torch.float16),
+    (1024, 512, 128, 256, 128, 6, 16, torch.bfloat16),
+    (512, 1024, 128, 128, 256, 2, 24, torch.bfloat16),
+    (640, 384, 96, 128, 128, 3, 32, torch.float16),
+    (768, 320, 160, 256, 64, 4, 256, torch.bfloat16),
+    (320, 192, 64, 64, 64, 1, 7, torch.bfloat16),
+    (300, 200, 72, 256, 256, 4, 8, torch.bfloat16),     # ragged M, N; K not a multiple of 32
+    (300, 200, 72, 128, 64, 4, 8, torch.float16),
+    (1, 1376, 256, 256, 256, 4, 256, torch.bfloat16),   # decoder shapes: one token, ragged N
+    (16, 1376, 512, 256, 64, 4, 256, torch.bfloat16),
+    (128, 1376, 1376, 256, 256, 4, 256, torch.bfloat16),  # ragged K tail of 32
+    (96, 80, 40, 32, 32, 2, 5, torch.bfloat16),         # logical tile smaller than any compute tile
+    (200, 136, 264, 96, 72, 2, 8, torch.bfloat16),      # logical tile no compute tile divides
+]
+
+
+@pytest.mark.parametrize("M,N,K,BM,BN,G,grid,dtype", SCATTER_CASES)
+def test_all_scatter_single_rank(shmem, M, N, K, BM, BN, G, grid, dtype):
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.full((M, N), 7, dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total + 3,), dtype=torch.int32)
+    ops.gemm_launch(a, b, None, cg, flags, shmem.get_heap_bases(), 0, 1, grid, BM, BN, 64, G,
+                    ops.EPI_ALL_SCATTER, num_xcds=ops.default_num_xcds(256, grid))
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, dtype), "all_scatter")
+    # one ready flag per tile, exactly one arrival each; nothing past the last tile
+    assert flags.cpu().tolist() == [1] * total + [0, 0, 0]
+
+
+def test_all_scatter_without_notify_leaves_flags_alone(shmem):
+    A, B = make_ab(256, 256, 64, torch.bfloat16)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((256, 256), dtype=torch.bfloat16)
+    flags = shmem.zeros((1,), dtype=torch.int32)
+    ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 4, 256, 256, 64, 4, ops.EPI_ALL_SCATTER, notify=False)
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, torch.bfloat16))
+    assert flags.cpu().tolist() == [0]
+
+
+@pytest.mark.parametrize("ws", [2, 8])
+def test_all_scatter_virtual_ranks(shmem, ws):
+    """N-split over ws ranks: rank r's [M, N/ws] block lands at column offset
+    r*N/ws of c_global on *every* rank; each rank's flags count ws arrivals."""
+    M, N, K, BM, BN, G = 256, 128 * ws, 128, 128, 64, 4
+    dtype = torch.bfloat16
+    A, B = make_ab(M, N, K, dtype)
+    shards = O.n_shards(A, B, ws)
+    a = to_heap(shmem, A)
+    bs = [to_heap(shmem, sb) for _, sb in shards]
+    cg = shmem.zeros((M, N), dtype=dtype)
+    n_local = N // ws
+    total = ops.cdiv(M, BM) * ops.cdiv(n_local, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    for r in range(ws):
+        shmem.on_rank(cg, r).zero_()
+        shmem.on_rank(flags, r).zero_()
+    for r in range(ws):
+        ops.gemm_launch(a, bs[r], None, shmem.on_rank(cg, r), shmem.on_rank(flags, r), shmem.get_heap_bases(), r,
+                        ws, 16, BM, BN, 64, G, ops.EPI_ALL_SCATTER)
+    torch.cuda.synchronize()
+    want = O.all_scatter(shards, dtype)
+    for r in range(ws):
+        check_close(shmem.on_rank(cg, r), want, f"rank {r}")
+        assert shmem.on_rank(flags, r).cpu().tolist() == [ws] * total
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_k_shard_views_keep_full_k_leading_dimension(shmem, dtype):
+    """The 08/09 sharding hands the kernel strided views of the full-K operands."""
+    M, N, K, ws = 384, 256, 512, 4
+    A, B = make_ab(M, N, K, dtype)
+    a_full, b_full = to_heap(shmem, A), to_heap(shmem, B)
+    ks = K // ws
+    cg = shmem.zeros((M, N), dtype=dtype)
+    flags = shmem.zeros((6,), dtype=torch.int32)
+    for r in (0, 3):
+        la, lb = a_full[:, r * ks:(r + 1) * ks], b_full[r * ks:(r + 1) * ks, :]
+        assert la.stride() == (K, 1) and lb.stride() == (1, K)
+        flags.zero_()
+        ops.gemm_launch(la, lb, None, cg, flags, None, 0, 1, 6, 128, 128, 64, 2, ops.EPI_ALL_SCATTER)
+        torch.cuda.synchronize()
+        check_close(cg, O.shard_gemm(A[:, r * ks:(r + 1) * ks], B[r * ks:(r + 1) * ks, :], dtype), f"shard {r}")
+
+
+def test_operands_the_dma_loader_cannot_take_use_the_generic_loader(shmem):
+    dtype = torch.bfloat16
+    # K not a multiple of 8
+    A, B = make_ab(130, 70, 100, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((130, 70), dtype=dtype)
+    ops.gemm_launch(a, b, None, cg, None, None, 0, 1, 4, 64, 64, 64, 2, ops.EPI_ALL_SCATTER, notify=False)
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, dtype), "K=100")
+    # A stored column-major (stride_ak != 1) and B row-major (stride_bk != 1)
+    g = torch.Generator().manual_seed(5)
+    At = (torch.randn(64, 96, generator=g) * 0.05).to(dtype)   # [K, M] storage
+    Bt = (torch.randn(64, 80, generator=g) * 0.05).to(dtype)   # [K, N] storage, row-major
+    a2 = shmem.zeros((64, 96), dtype=dtype)
+    a2.copy_(At)
+    b2 = shmem.zeros((64, 80), dtype=dtype)
+    b2.copy_(Bt)
+    cg2 = shmem.zeros((96, 80), dtype=dtype)
+    ops.gemm_launch(a2.T, b2, None, cg2, None, None, 0, 1, 4, 64, 64, 64, 2, ops.EPI_ALL_SCATTER, notify=False)
+    torch.cuda.synchronize()
+    check_close(cg2, O.shard_gemm(At.T, Bt, dtype), "transposed operands")
+    # K == 0: the product is all zeros
+    cg3 = shmem.full((96, 80), 3, dtype=dtype)
+    ops.gemm_launch(a2.T[:, :0], b2[:0, :], None, cg3, None, None, 0, 1, 4, 64, 64, 64, 2, ops.EPI_ALL_SCATTER,
+                    notify=False)
+    torch.cuda.synchronize()
+    assert float(cg3.float().abs().max()) == 0.0
+
+
+def test_unaligned_and_strided_output(shmem):
+    dtype = torch.bfloat16
+    A, B = make_ab(256, 192, 64, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    big = shmem.zeros((256, 200), dtype=dtype)
+    cg = big[:, 3:195]  # column offset 3: rows are not 16-byte aligned
+    ops.gemm_launch(a, b, None, cg, None, None, 0, 1, 4, 128, 64, 64, 2, ops.EPI_ALL_SCATTER, notify=False)
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, dtype))
+    assert float(big[:, :3].float().abs().max()) == 0.0 and float(big[:, 195:].float().abs().max()) == 0.0
+    cgt = shmem.zeros((192, 256), dtype=dtype).T  # column-major result
+    ops.gemm_launch(a, b, None, cgt, None, None, 0, 1, 4, 128, 64, 64, 2, ops.EPI_ALL_SCATTER, notify=False)
+    torch.cuda.synchronize()
+    check_close(cgt, O.shard_gemm(A, B, dtype))
+    c32 = shmem.zeros((256, 192), dtype=torch.float32)  # fp32 destination
+    ops.gemm_launch(a, b, None, c32, None, None, 0, 1, 4, 128, 64, 64, 2, ops.EPI_ALL_SCATTER, notify=False)
+    torch.cuda.synchronize()
+    check_close(c32, O.shard_gemm(A, B, None))
+
+
+@pytest.mark.parametrize("variant", range(1, 11))
+def test_every_tuning_variant_is_correct(shmem, variant):
+    """Each compiled kernel variant of the bf16 store path, forced on a shape
+    with ragged edges and several tiles per program."""
+    name = ops.gemm_variant_name(torch.bfloat16, False, False, variant)
+    assert name is not None
+    dtype = torch.bfloat16
+    M, N, K = 520, 776, 328
+    A, B = make_ab(M, N, K, dtype, lda=336, ldb=344)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, 256) * ops.cdiv(N, 256)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 5, 256, 256, 64, 2, ops.EPI_ALL_SCATTER, variant=variant)
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, dtype), name)
+    assert flags.cpu().tolist() == [1] * total
+    assert ops.gemm_variant_name(torch.bfloat16, False, False, 11) is None
+
+
+# --------------------------------------------------------------------------- atomics
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_atomic_accumulate_of_eight_k_shards(shmem, out_dtype):
+    """Eight sequential shard GEMMs, each adding its tiles into one shared C."""
+    M, N, K, ws = 512, 384, 1024, 8
+    dtype = torch.bfloat16
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    a_full, b_full = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((M, N), dtype=out_dtype)
+    ks = K // ws
+    for r in range(ws):
+        ops.gemm_launch(a_full[:, r * ks:(r + 1) * ks], b_full[r * ks:(r + 1) * ks, :], None, cg, None, None, 0, 1,
+                        8, 256, 128, 64, 6, ops.EPI_ATOMIC_ADD)
+    torch.cuda.synchronize()
+    want = O.atomics_all_reduce(O.k_shards(A, B, ws))
+    if out_dtype == torch.float32:
+        check_close(cg, want, "fp32 atomics")
+    else:
+        # 16-bit accumulation rounds after every add: 8 roundings of half an ulp each
+        err = (cg.float().cpu() - want).abs()
+        assert float(err.max()) <= 8 * 2.0 ** -8 * float(want.abs().max()) + ATOL
+
+
+def test_atomic_add_ragged_and_on_every_rank(shmem):
+    M, N, K, ws = 200, 136, 96, 2
+    dtype = torch.float16
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((M, N), dtype=torch.float32)
+    for r in range(ws):
+        shmem.on_rank(cg, r).fill_(1.0)
+    # rank 1 adds its product into c_global of both ranks
+    ops.gemm_launch(a, b, None, shmem.on_rank(cg, 1), None, shmem.get_heap_bases(), 1, ws, 4, 128, 64, 64, 2,
+                    ops.EPI_ATOMIC_ADD)
+    torch.cuda.synchronize()
+    want = O.shard_gemm(A, B, None) + 1.0
+    for r in range(ws):
+        check_close(shmem.on_rank(cg, r), want, f"rank {r}")
+
+
+# --------------------------------------------------------------------------- one-shot
+@pytest.mark.parametrize("partial_dtype", [torch.bfloat16, torch.float32])
+def test_one_shot_fused_single_rank(shmem, partial_dtype):
+    """world_size 1: store the tile to C, no flag traffic, c_global = cast(C)."""
+    M, N, K = 384, 320, 192
+    dtype = torch.bfloat16
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    c = shmem.zeros((M, N), dtype=partial_dtype)
+    cg = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, 128) * ops.cdiv(N, 64)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    ops.gemm_launch(a, b, c, cg, flags, shmem.get_heap_bases(), 0, 1, 8, 128, 64, 64, 6, ops.EPI_ONE_SHOT,
+                    phase=ops.PHASE_FUSED)
+    torch.cuda.synchronize()
+    check_close(c, O.shard_gemm(A, B, partial_dtype), "partial")
+    assert torch.equal(cg.cpu(), O.one_shot_reduce(c.cpu()[None], dtype))  # bit-exact given the partial
+    assert flags.cpu().tolist() == [0] * total  # ws == 1: no flag is ever written
+
+
+@pytest.mark.parametrize("ws,partial_dtype", [(2, torch.bfloat16), (8, torch.float32), (8, torch.float16)])
+def test_one_shot_all_reduce_virtual_ranks(shmem, ws, partial_dtype):
+    """K-split over ws ranks on one GPU: every rank produces (partial tile +
+    signal), then every rank consumes (wait, reduce, store)."""
+    M, N, K, BM, BN, G = 256, 320, 64 * ws, 128, 64, 6
+    dtype = torch.float16 if partial_dtype == torch.float16 else torch.bfloat16
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    a_full, b_full = to_heap(shmem, A), to_heap(shmem, B)
+    ks = K // ws
+    c = shmem.zeros((M, N), dtype=partial_dtype)
+    cg = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for r in range(ws):
+        for t in (c, cg, flags):
+            shmem.on_rank(t, r).zero_()
+    hb = shmem.get_heap_bases()
+
+    def launch(r, phase):
+        ops.gemm_launch(a_full[:, r * ks:(r + 1) * ks], b_full[r * ks:(r + 1) * ks, :], shmem.on_rank(c, r),
+                        shmem.on_rank(cg, r), shmem.on_rank(flags, r), hb, r, ws, 8, BM, BN, 64, G,
+                        ops.EPI_ONE_SHOT, phase=phase, status=status)
+
+    for r in range(ws):
+        launch(r, ops.PHASE_PRODUCE)
+    torch.cuda.synchronize()
+    fm = O.FlagModel(ws, total)
+    for r in range(ws):
+        for t in range(total):
+            fm.signal(r, t)
+    for r in range(ws):  # every producer added +1 on every *other* rank
+        assert shmem.on_rank(flags, r).cpu().tolist() == fm.flags[r].tolist() == [ws - 1] * total
+    partials = torch.stack([shmem.on_rank(c, r).cpu() for r in range(ws)])
+    shards = O.k_shards(A, B, ws)
+    for r in range(ws):
+        check_close(partials[r], O.shard_gemm(*shards[r], partial_dtype), f"partial {r}")
+    for r in range(ws):
+        launch(r, ops.PHASE_CONSUME)
+    torch.cuda.synchronize()
+    want_bits = O.one_shot_reduce(partials, dtype)
+    for r in range(ws):
+        assert torch.equal(shmem.on_rank(cg, r).cpu(), want_bits), f"rank {r}"  # fixed rank order: bit-exact
+        assert shmem.on_rank(flags, r).cpu().tolist() == [0] * total            # the CAS resets every flag
+    check_close(cg, O.one_shot_all_reduce(shards, partial_dtype, dtype), "vs closed form")
+    assert int(status.item()) == 0
+
+
+def test_fused_phase_with_peers_missing_times_out_and_exits(shmem):
+    """A rank whose peers never signal: the bounded wait gives up, reports it
+    and skips the reduce; the kernel still drains."""
+    M, N, K, ws = 128, 128, 64, 2
+    dtype = torch.bfloat16
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    c = shmem.zeros((M, N), dtype=dtype)
+    cg = shmem.full((M, N), 5, dtype=dtype)
+    flags = shmem.zeros((4,), dtype=torch.int32)
+    for r in range(ws):
+        shmem.on_rank(flags, r).zero_()
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ops.gemm_launch(a, b, c, cg, flags, shmem.get_heap_bases(), 0, ws, 4, 64, 64, 64, 1, ops.EPI_ONE_SHOT,
+                    phase=ops.PHASE_FUSED, status=status, spin_timeout_ticks=2000)  # 20 us
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+    assert float((cg.float() - 5).abs().max()) == 0.0  # nothing was reduced
+    check_close(c, O.shard_gemm(A, B, dtype))           # the partial was still produced
+    assert shmem.on_rank(flags, 1).cpu().tolist() == [1] * 4 and flags.cpu().tolist() == [0] * 4
+
+
+# --------------------------------------------------------------------------- schedule, timestamps, registers
+@pytest.mark.parametrize("M,N,BM,BN,G,num_sms,x", [
+    (8192, 8192, 256, 256, 4, 256, 8), (8192, 8192, 256, 256, 6, 256, 1), (4096, 4096, 256, 256, 6, 288, 8),
+    (2048, 1376, 256, 64, 4, 304, 8), (1, 1376, 256, 256, 4, 256, 8), (1000, 999, 64, 64, 5, 56, 4),
+])
+def test_device_tile_schedule_is_bit_exact(M, N, BM, BN, G, num_sms, x):
+    got = ops.tile_schedule(M, N, BM, BN, G, num_sms, x).cpu().numpy()
+    total = O.cdiv(M, BM) * O.cdiv(N, BN)
+    want = np.full((total, 4), -1, dtype=np.int32)
+    want[:, :2] = O.tile_map_all(M, N, BM, BN, G)
+    for p in range(num_sms):
+        for pos, t in enumerate(O.program_tiles(p, total, num_sms, x)):
+            want[t, 2:] = (p, pos)
+    assert (got == want).all()
+
+
+def test_tile_timestamps_and_kernel_info(shmem):
+    M, N, K = 512, 512, 128
+    dtype = torch.bfloat16
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((M, N), dtype=dtype)
+    total = 16
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    begin = torch.full((total,), torch.iinfo(torch.int64).max, dtype=torch.int64, device="cuda")
+    end = torch.zeros(total, dtype=torch.int64, device="cuda")
+    ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 2, 128, 128, 64, 2, ops.EPI_ALL_SCATTER,
+                    mm_begin_timestamp=begin, mm_end_timestamp=end)
+    torch.cuda.synchronize()
+    bg, en = begin.cpu(), end.cpu()
+    assert (bg < torch.iinfo(torch.int64).max).all() and (en > 0).all() and (bg <= en).all()
+    # program 0 walks tiles 0, 2, 4, ... in order
+    mine = bg[0::2]
+    assert (mine[1:] >= mine[:-1]).all()
+    check_close(cg, O.shard_gemm(A, B, dtype))
+    regs, spills = ops.gemm_kernel_info(a, b, None, cg, flags, None, 0, 1, 2, 128, 128, 64, 2, ops.EPI_ALL_SCATTER)
+    assert 0 < regs <= 512 and spills == 0
+
+
+def test_launcher_rejects_what_the_kernels_do_not_take(shmem):
+    A, B = make_ab(64, 64, 64, torch.bfloat16)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((64, 64), dtype=torch.bfloat16)
+    with pytest.raises(ValueError):  # c_global too small for two ranks' columns
+        ops.gemm_launch(a, b, None, cg, None, shmem.get_heap_bases(), 0, 2, 4, 64, 64, 64, 1, ops.EPI_ALL_SCATTER,
+                        notify=False)
+    with pytest.raises(ValueError):  # too few flags
+        ops.gemm_launch(a, b, None, cg, shmem.zeros((0,), dtype=torch.int32), None, 0, 1, 4, 32, 32, 64, 1,
+                        ops.EPI_ALL_SCATTER)
+    with pytest.raises(ValueError):  # grid does not split over the XCDs
+        ops.gemm_launch(a, b, None, cg, None, None, 0, 1, 12, 64, 64, 64, 1, ops.EPI_ALL_SCATTER, notify=False,
+                        num_xcds=8)
+    with pytest.raises(ValueError):  # fp16 result from bf16 operands
+        ops.gemm_launch(a, b, None, shmem.zeros((64, 64), dtype=torch.float16), None, None, 0, 1, 4, 64, 64, 64, 1,
+                        ops.EPI_ALL_SCATTER, notify=False)
+    with pytest.raises(TypeError):  # fp32 operands
+        ops.gemm_launch(a.float(), b.float(), None, cg, None, None, 0, 1, 4, 64, 64, 64, 1, ops.EPI_ALL_SCATTER,
+                        notify=False)
