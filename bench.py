@@ -115,8 +115,8 @@ def main():
         sys.exit(1)
 
     ws = 8
-    # per-rank heap: 256 MiB fp32 partial + 128 MiB bf16 result + operands/flags
-    shmem = iris_amd.iris(480 << 20, virtual_ranks=ws)
+    # per-rank heap: full-K operands 2 x 128 MiB, bf16 results 2 x 128 MiB, fp32 partial 256 MiB, flags
+    shmem = iris_amd.iris(1 << 30, virtual_ranks=ws)
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(123)
     # one rank's K-shard as a strided view of the full-K operands (the 08/09 sharding)

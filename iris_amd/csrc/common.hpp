@@ -58,6 +58,13 @@ __host__ __device__ inline int xcd_remap(int pid, int num_sms, int num_xcds) {
   return pid;
 }
 
+// A 64-bit value every lane of the wave agrees on, as scalar registers.
+__device__ inline uint64_t uniform_u64(uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
 // Pointer rebasing between symmetric heaps; iris/iris.py:317-339.
 template <typename P>
 __device__ inline IRIS_GLOBAL P* translate(P* ptr, uint64_t cur_base, uint64_t target_base) {
@@ -126,6 +133,23 @@ __device__ inline void flag_add_release(IRIS_GLOBAL int32_t* p, int v, bool sys)
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   else
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ inline void flag_add_relaxed(IRIS_GLOBAL int32_t* p, int v, bool sys) {
+  if (sys)
+    __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  else
+    __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Store that is written through to the coherence point of the agent (or of
+// the system): nothing stays dirty in this XCD's L2.
+template <typename T>
+__device__ inline void store_through(IRIS_GLOBAL T* p, T v, bool sys) {
+  if (sys)
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  else
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // CAS(expected -> desired) with acquire; returns the old value

@@ -15,13 +15,22 @@
 //   * v_mfma_f32_32x32x16 (bf16 or f16) with fp32 accumulators; operands are
 //     swapped (B rows as SrcA, A rows as SrcB) so that a lane ends up with 4
 //     consecutive columns of one output row.
+//   * Operand fragments are fetched from LDS one K-substep (16 k) ahead of
+//     the MFMAs that use them, and the barrier that hands over the next
+//     stage sits in the middle of a step's MFMA stream, so neither LDS
+//     latency nor the barrier is paid with idle matrix cores.
 //   * The epilogue transposes the accumulators through a wave-private LDS
 //     scratch so that global stores / atomics cover contiguous row segments.
+//     Stores are write-through at the flags' scope; once they have completed
+//     nothing is left in L2 for a release to write back, and a tile's flag is
+//     published with a relaxed atomic.
 //
 // The logical tile (BLOCK_SIZE_M x BLOCK_SIZE_N, which fixes tile ids and
 // flags) may be larger than the compute tile (CM x CN); a logical tile is
 // then covered by several compute tiles and published once.
 #pragma once
+
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -91,7 +100,10 @@ struct GemmCfg {
   static_assert((CM * CPR) % NT == 0 && (CN * CPR) % NT == 0, "slab must split evenly over lanes");
   static_assert(A_LOADS >= 1 && B_LOADS >= 1, "too many waves for this slab");
   static_assert((S & (S - 1)) == 0 && S >= 1, "ring depth must be a power of two");
+  static_assert(!DMA || S >= 4, "the DMA ring needs a stage being refilled, read, landed and in flight");
   static_assert(L * (S > 2 ? S - 2 : 0) <= 63, "vmcnt immediate");
+  static_assert(KSUB % 2 == 0, "fragment double-buffering alternates per K-substep");
+  static_assert(RPB % (RP * CPR) == 0, "XOR term of a DMA block must depend on the lane only");
   static_assert(TN == 32 || TN == 64 || TN == 128, "wave tile width");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
@@ -130,7 +142,8 @@ __device__ inline Item decode_item(const GemmKArgs& p, int pid, int item) {
 template <typename P>
 __device__ inline IRIS_GLOBAL P* rank_ptr(const GemmKArgs& p, P* ptr, int r) {
   if (r == p.cur_rank || p.heap_bases == nullptr) return (IRIS_GLOBAL P*)ptr;
-  return translate(ptr, p.heap_bases[p.cur_rank], p.heap_bases[r]);
+  // r and the bases are the same for the whole wave: keep the result scalar
+  return translate(ptr, uniform_u64(p.heap_bases[p.cur_rank]), uniform_u64(p.heap_bases[r]));
 }
 
 // ---------------------------------------------------------------------------
@@ -145,7 +158,7 @@ template <class Cfg>
 struct Loader {
   __amdgpu_buffer_rsrc_t ra, rb;
   uint32_t voff[Cfg::L];  // byte offset of (row, logical chunk) at k0 == 0
-  uint32_t kcol[Cfg::L];  // first k of the chunk at k0 == 0
+  int kcol;               // first k of this lane's chunk at k0 == 0 (the same for every load)
 
   __device__ inline void setup(const GemmKArgs& p, const Item& it, int wave, int lane) {
     // Rows past the matrix edge re-read the last valid row (the reference
@@ -158,32 +171,34 @@ struct Loader {
     const uint32_t brec = (uint32_t)(((int64_t)(rows_b - 1) * p.sbn + p.K) * 2);
     ra = __builtin_amdgcn_make_buffer_rsrc((void*)abase, 0, arec, 0x00020000);
     rb = __builtin_amdgcn_make_buffer_rsrc((void*)bbase, 0, brec, 0x00020000);
+    // a 1 KiB block holds RPB = RP*CPR*k rows, so the row's XOR term depends
+    // on the lane only
+    const int ch = (lane % Cfg::CPR) ^ (((lane / Cfg::CPR) / Cfg::RP) % Cfg::CPR);
+    kcol = ch * 8;
 #pragma unroll
     for (int i = 0; i < Cfg::L; ++i) {
       const bool isA = i < Cfg::A_LOADS;
       const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
       const int row = blk * Cfg::RPB + lane / Cfg::CPR;
-      const int pc = lane % Cfg::CPR;
-      const int ch = pc ^ ((row / Cfg::RP) % Cfg::CPR);
       const int rclamp = min(row, (isA ? rows_a : rows_b) - 1);
       const int64_t ld = isA ? p.sam : p.sbn;
       voff[i] = (uint32_t)(((int64_t)rclamp * ld + ch * 8) * 2);
-      kcol[i] = ch * 8;
     }
   }
 
   // Issue the L loads of K-step `k` into the stage at LDS address `stage`.
   __device__ inline void issue(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
     const int k0 = k * Cfg::BK;
+    // chunks past K read as zero: an offset beyond num_records is out of
+    // range for the buffer and the load returns 0 (the masked tail of
+    // gemm_*:186-195)
+    const bool in_k = k0 + kcol < p.K;
 #pragma unroll
     for (int i = 0; i < Cfg::L; ++i) {
       const bool isA = i < Cfg::A_LOADS;
       const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
       IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + blk * 1024;
-      // chunks past K read as zero: an offset beyond num_records is out of
-      // range for the buffer and the load returns 0 (the masked tail of
-      // gemm_*:186-195)
-      const uint32_t off = ((int)(k0 + kcol[i]) < p.K) ? voff[i] + (uint32_t)k0 * 2 : 0x80000000u;
+      const uint32_t off = in_k ? voff[i] + (uint32_t)k0 * 2 : 0x80000000u;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, 0, 0, 0);
     }
   }
@@ -231,39 +246,38 @@ __device__ inline void load_slab_generic(const GemmKArgs& p, const Item& it, IRI
 // MFMA over one stage
 // ---------------------------------------------------------------------------
 
-template <class Cfg, bool FIRST>
-__device__ inline void compute_stage(const IRIS_LDS char* stage, f32x16 (&acc)[Cfg::IM][Cfg::IN], int a_row_off,
-                                     int b_row_off, const int (&xoff)[Cfg::KSUB]) {
+template <class Cfg>
+struct Frags {
+  typename Mfma<Cfg::DT>::vec8 a[Cfg::IM], b[Cfg::IN];
+};
+
+// Fetch the operand fragments of one K-substep (16 k) of a stage.
+template <class Cfg>
+__device__ inline void load_frags(const IRIS_LDS char* stage, int a_row_off, int b_row_off, int xo, Frags<Cfg>& f) {
   using V = typename Mfma<Cfg::DT>::vec8;
-  const IRIS_LDS char* sA = stage + a_row_off;
-  const IRIS_LDS char* sB = stage + Cfg::A_BYTES + b_row_off;
-  // all operand fragments of the K-step are requested up front; the MFMAs
-  // then start as the first ones arrive (LDS returns in order)
-  V a[Cfg::KSUB][Cfg::IM], b[Cfg::KSUB][Cfg::IN];
+  const IRIS_LDS char* sA = stage + a_row_off + xo;
+  const IRIS_LDS char* sB = stage + Cfg::A_BYTES + b_row_off + xo;
 #pragma unroll
-  for (int kk = 0; kk < Cfg::KSUB; ++kk) {
+  for (int j = 0; j < Cfg::IN; ++j) f.b[j] = *reinterpret_cast<const IRIS_LDS V*>(sB + j * 32 * Cfg::BK * 2);
 #pragma unroll
-    for (int j = 0; j < Cfg::IN; ++j)
-      b[kk][j] = *reinterpret_cast<const IRIS_LDS V*>(sB + j * 32 * Cfg::BK * 2 + xoff[kk]);
+  for (int i = 0; i < Cfg::IM; ++i) f.a[i] = *reinterpret_cast<const IRIS_LDS V*>(sA + i * 32 * Cfg::BK * 2);
+}
+
+// acc (+)= B-fragment x A-fragment for every 32x32 block of the wave tile.
+// FIRST starts a tile: the accumulator input is the constant 0.
+template <class Cfg, bool FIRST>
+__device__ inline void mma_frags(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& f) {
 #pragma unroll
-    for (int i = 0; i < Cfg::IM; ++i)
-      a[kk][i] = *reinterpret_cast<const IRIS_LDS V*>(sA + i * 32 * Cfg::BK * 2 + xoff[kk]);
-  }
-  __builtin_amdgcn_sched_barrier(0);  // keep the fetches ahead of the MFMAs
+  for (int i = 0; i < Cfg::IM; ++i)
 #pragma unroll
-  for (int kk = 0; kk < Cfg::KSUB; ++kk) {
-#pragma unroll
-    for (int i = 0; i < Cfg::IM; ++i)
-#pragma unroll
-      for (int j = 0; j < Cfg::IN; ++j) {
-        if (FIRST && kk == 0) {
-          const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-          acc[i][j] = Mfma<Cfg::DT>::run(b[kk][j], a[kk][i], z);
-        } else {
-          acc[i][j] = Mfma<Cfg::DT>::run(b[kk][j], a[kk][i], acc[i][j]);
-        }
+    for (int j = 0; j < Cfg::IN; ++j) {
+      if (FIRST) {
+        const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        acc[i][j] = Mfma<Cfg::DT>::run(f.b[j], f.a[i], z);
+      } else {
+        acc[i][j] = Mfma<Cfg::DT>::run(f.b[j], f.a[i], acc[i][j]);
       }
-  }
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -386,14 +400,27 @@ __device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM
             }
           } else {
             constexpr int RPI = 64 / Cfg::U16;  // rows per wave-wide 16-byte read
+            constexpr int NV = 32 / RPI;
+            // the 32 x CP block as a buffer: rows are p.som elements apart
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+                (void*)(dst + ((int64_t)row0 * p.som + col0) * ES), 0, (int)((31 * p.som + CP) * ES), 0x00020000);
+            u32x4 v[NV];
+            int off[NV];
 #pragma unroll
-            for (int t = 0; t < 32 / RPI; ++t) {
+            for (int t = 0; t < NV; ++t) {
               const int row = t * RPI + lane / Cfg::U16;
               const int u = lane % Cfg::U16;
               const int pu = u ^ ((row / Cfg::ERPB) % Cfg::U16);
-              const u32x4 v = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + row * Cfg::WS_PITCH + pu * 16);
-              const int m = row0 + row, n = col0 + u * EPV;
-              *(IRIS_GLOBAL u32x4*)(dst + ((int64_t)m * p.som + n) * ES) = v;
+              v[t] = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + row * Cfg::WS_PITCH + pu * 16);
+              off[t] = (int)((row * p.som + u * EPV) * ES);
+            }
+            // write-through at the flags' scope: sc1 (agent) or sc0 sc1 (system)
+            if (p.sys) {
+#pragma unroll
+              for (int t = 0; t < NV; ++t) __builtin_amdgcn_raw_buffer_store_b128(v[t], rs, off[t], 0, 17);
+            } else {
+#pragma unroll
+              for (int t = 0; t < NV; ++t) __builtin_amdgcn_raw_buffer_store_b128(v[t], rs, off[t], 0, 16);
             }
           }
         } else {
@@ -407,9 +434,11 @@ __device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM
             if (m < m_end && n < n_end) {
               IRIS_GLOBAL char* d = dst + ((int64_t)m * p.som + (int64_t)n * p.son) * ES;
               if constexpr (OP == OP_STORE32)
-                *(IRIS_GLOBAL unsigned int*)d = *reinterpret_cast<const IRIS_LDS unsigned int*>(src);
+                store_through((IRIS_GLOBAL unsigned int*)d, *reinterpret_cast<const IRIS_LDS unsigned int*>(src),
+                              p.sys != 0);
               else if constexpr (OP == OP_STORE16)
-                *(IRIS_GLOBAL unsigned short*)d = *reinterpret_cast<const IRIS_LDS unsigned short*>(src);
+                store_through((IRIS_GLOBAL unsigned short*)d,
+                              *reinterpret_cast<const IRIS_LDS unsigned short*>(src), p.sys != 0);
               else
                 atomic_add16_cas<ODT>((IRIS_GLOBAL unsigned short*)d,
                                       from16<ODT>(*reinterpret_cast<const IRIS_LDS unsigned short*>(src)));
@@ -421,16 +450,19 @@ __device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM
   }
 }
 
-// Publish a finished logical tile: +1 (release) on the tile's flag of every
-// rank (flag_mode 1, the ready flag of the scatter epilogue) or of every
-// *other* rank (flag_mode 2, the ONE_SHOT producer signal,
-// gemm_one_shot_all_reduce.py:207-218).  One thread; the caller has made
-// every wave's stores complete and passed a barrier.
+// Publish a finished logical tile: +1 on the tile's flag of every rank
+// (flag_mode 1, the ready flag of the scatter epilogue) or of every *other*
+// rank (flag_mode 2, the ONE_SHOT producer signal,
+// gemm_one_shot_all_reduce.py:207-218, sem="release").  One thread calls it
+// after every wave of the group has waited for its stores of the tile to
+// complete and the group has passed a barrier.  Those stores were
+// write-through at the flag's scope, so they are already visible there and
+// the increment itself can be relaxed: it is ordered after them by the waits.
 __device__ inline void publish_tile(const GemmKArgs& p, int tile_id) {
 #pragma nounroll
   for (int r = 0; r < p.ws; ++r) {
     if (p.flag_mode == 2 && r == p.cur_rank) continue;
-    flag_add_release(rank_ptr(p, p.flags + tile_id, r), 1, p.sys != 0);
+    flag_add_relaxed(rank_ptr(p, p.flags + tile_id, r), 1, p.sys != 0);
   }
 }
 
@@ -479,79 +511,12 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArg
   const bool defer_publish = Cfg::DMA && nk > 0 && p.flag_mode != 0;
   int pending_tile = -1;
 
-  Loader<Cfg> ld;
-  int l_item = 0, l_k = 0;  // load cursor
-  Item l_it;
-  if (Cfg::DMA && total_steps > 0) {
-    l_it = decode_item<Cfg>(p, pid, 0);
-    ld.setup(p, l_it, wave, lane);
-#pragma unroll
-    for (int s = 0; s < Cfg::S - 1; ++s) {
-      if (s < total_steps) {
-        ld.issue(p, lds + s * Cfg::STAGE, l_k, wave);
-        if (++l_k == nk) {
-          l_k = 0;
-          ++l_item;
-          if (l_item < n_items) {
-            l_it = decode_item<Cfg>(p, pid, l_item);
-            ld.setup(p, l_it, wave, lane);
-          }
-        }
-      }
-    }
-  }
-
   int c_item = 0, c_k = 0;  // compute cursor
   Item c_it;
   if (n_items > 0) c_it = decode_item<Cfg>(p, pid, 0);
 
-  // K == 0 leaves every tile all zeros: one epilogue per item, no loads.
-  const int n_outer = nk > 0 ? total_steps : n_items;
-  for (int g = 0; g < n_outer; ++g) {
-    if (nk > 0) {
-      IRIS_LDS char* stage = lds + (Cfg::DMA ? (g & (Cfg::S - 1)) : 0) * Cfg::STAGE;
-      if constexpr (Cfg::DMA) {
-        // wait for this step's slab; S-2 younger slabs may stay in flight
-        if (pending_tile >= 0 || g + Cfg::S - 2 > total_steps - 1 || Cfg::S < 3) {
-          IRIS_WAIT_VMCNT(0);
-        } else {
-          IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S > 2 ? Cfg::S - 2 : 0));
-        }
-        block_barrier_raw();  // slab visible to all waves; previous slab's readers done
-        if (pending_tile >= 0) {
-          if (tid == 0) publish_tile(p, pending_tile);
-          pending_tile = -1;
-        }
-        if (g + Cfg::S - 1 < total_steps) {
-          ld.issue(p, lds + ((g + Cfg::S - 1) & (Cfg::S - 1)) * Cfg::STAGE, l_k, wave);
-          if (++l_k == nk) {
-            l_k = 0;
-            ++l_item;
-            if (l_item < n_items) {
-              l_it = decode_item<Cfg>(p, pid, l_item);
-              ld.setup(p, l_it, wave, lane);
-            }
-          }
-        }
-      } else {
-        __syncthreads();  // previous step's readers are done with the stage
-        load_slab_generic<Cfg>(p, c_it, stage, c_k, tid);
-        __syncthreads();
-      }
-
-      if (c_k == 0) {
-        if (p.ts_begin && c_it.first_sub && tid == 0)
-          __hip_atomic_fetch_min((IRIS_GLOBAL unsigned long long*)(p.ts_begin + c_it.tile_id),
-                                 (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        compute_stage<Cfg, true>(stage, acc, a_row_off, b_row_off, xoff);
-      } else {
-        compute_stage<Cfg, false>(stage, acc, a_row_off, b_row_off, xoff);
-      }
-      if (++c_k < nk) continue;
-      c_k = 0;
-    }
-
-    // ---------------- epilogue of one compute tile ----------------
+  // end of a compute tile: store it, and publish the logical tile it completes
+  auto epilogue = [&]() __attribute__((always_inline)) {
     store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end, c_it.n_end,
                             lane);
     if (c_it.last_sub) {
@@ -567,6 +532,120 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArg
                                (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (++c_item < n_items) c_it = decode_item<Cfg>(p, pid, c_item);
+  };
+  auto stamp_begin = [&]() __attribute__((always_inline)) {
+    if (p.ts_begin && c_it.first_sub && tid == 0)
+      __hip_atomic_fetch_min((IRIS_GLOBAL unsigned long long*)(p.ts_begin + c_it.tile_id),
+                             (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+
+  if (nk == 0) {
+    // K == 0 leaves every tile all zeros: one epilogue per item, no loads
+    for (int it = 0; it < n_items; ++it) epilogue();
+  } else if constexpr (Cfg::DMA) {
+    // ---- the flattened (item, k) pipeline -------------------------------
+    // Ring of S stages.  While step g is multiplied: stage g is being read,
+    // stage g+1 has landed, stage g+2 is in flight and stage g-1 is being
+    // refilled with step g+3.
+    Loader<Cfg> ld;
+    int l_item = 0, l_k = 0;  // load cursor
+    Item l_it;
+    auto issue_next = [&](IRIS_LDS char* stage) __attribute__((always_inline)) {
+      ld.issue(p, stage, l_k, wave);
+      if (++l_k == nk) {
+        l_k = 0;
+        if (++l_item < n_items) {
+          l_it = decode_item<Cfg>(p, pid, l_item);
+          ld.setup(p, l_it, wave, lane);
+        }
+      }
+    };
+    if (total_steps > 0) {
+      l_it = decode_item<Cfg>(p, pid, 0);
+      ld.setup(p, l_it, wave, lane);
+#pragma unroll
+      for (int s = 0; s < Cfg::S - 1; ++s)
+        if (s < total_steps) issue_next(lds + s * Cfg::STAGE);
+      // stage 0 has landed once at most S-2 younger slabs are outstanding
+      if (total_steps >= Cfg::S - 1) {
+        IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
+      } else {
+        IRIS_WAIT_VMCNT(0);
+      }
+      block_barrier_raw();
+    }
+    Frags<Cfg> fr[2];
+    if (total_steps > 0) load_frags<Cfg>(lds, a_row_off, b_row_off, xoff[0], fr[0]);
+
+    // One K-step.  LAST is the final step of the program: nothing is handed
+    // over or prefetched after it (kept out of the loop so that the loop body
+    // is straight-line code around its MFMAs).
+    auto step = [&](int g, auto last_tag) __attribute__((always_inline)) {
+      constexpr bool LAST = decltype(last_tag)::value;
+      const IRIS_LDS char* stage = lds + (g & (Cfg::S - 1)) * Cfg::STAGE;
+      if (c_k == 0) stamp_begin();
+#pragma unroll
+      for (int kk = 0; kk < Cfg::KSUB; ++kk) {
+        // fetch the next K-substep's fragments before multiplying this one
+        if (kk + 1 < Cfg::KSUB) {
+          load_frags<Cfg>(stage, a_row_off, b_row_off, xoff[kk + 1], fr[(kk + 1) & 1]);
+        } else if (!LAST) {
+          // hand-over of stage g+1: wait for this wave's part of its slab
+          // (S-3 younger slabs may stay in flight), then meet the other waves
+          if (pending_tile >= 0 || g + Cfg::S - 2 > total_steps - 1) {
+            IRIS_WAIT_VMCNT(0);
+          } else {
+            IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 3));
+          }
+          block_barrier_raw();
+          if (pending_tile >= 0) {
+            if (tid == 0) publish_tile(p, pending_tile);
+            pending_tile = -1;
+          }
+          // every wave is past its reads of stage g-1: refill it
+          if (g + Cfg::S - 1 < total_steps) issue_next(lds + ((g + Cfg::S - 1) & (Cfg::S - 1)) * Cfg::STAGE);
+          load_frags<Cfg>(lds + ((g + 1) & (Cfg::S - 1)) * Cfg::STAGE, a_row_off, b_row_off, xoff[0], fr[0]);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // fetches stay ahead of the MFMAs they overlap
+        if (kk == 0 && c_k == 0)
+          mma_frags<Cfg, true>(acc, fr[0]);
+        else
+          mma_frags<Cfg, false>(acc, fr[kk & 1]);
+        // The fragments requested above have had this whole MFMA block to
+        // arrive.  Waiting for them here costs nothing and spares the next
+        // block a wait that would also cover the requests issued just before it.
+        __builtin_amdgcn_sched_barrier(0);
+        IRIS_WAIT_LGKMCNT0();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (++c_k == nk) {
+        c_k = 0;
+        epilogue();
+      }
+    };
+    for (int g = 0; g < total_steps - 1; ++g) step(g, std::false_type{});
+    if (total_steps > 0) step(total_steps - 1, std::true_type{});
+  } else {
+    // ---- generic loader: one stage, synchronous ---------------------------
+    Frags<Cfg> fr;
+    for (int g = 0; g < total_steps; ++g) {
+      __syncthreads();  // previous step's readers are done with the stage
+      load_slab_generic<Cfg>(p, c_it, lds, c_k, tid);
+      __syncthreads();
+      if (c_k == 0) stamp_begin();
+#pragma unroll
+      for (int kk = 0; kk < Cfg::KSUB; ++kk) {
+        load_frags<Cfg>(lds, a_row_off, b_row_off, xoff[kk], fr);
+        if (kk == 0 && c_k == 0)
+          mma_frags<Cfg, true>(acc, fr);
+        else
+          mma_frags<Cfg, false>(acc, fr);
+      }
+      if (++c_k == nk) {
+        c_k = 0;
+        epilogue();
+      }
+    }
   }
 
   if (pending_tile >= 0) {
