@@ -55,15 +55,27 @@ struct GemmKArgs {
   int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
   int sys;           // flag atomics at system scope (else agent)
   int vec_out;       // 16-byte vector access allowed on `out`
+  int debug;         // tuning experiments only (IRIS_AMD_GEMM_DEBUG): 1 = fetch nothing, 2 = every row fetches row 0
 };
 
 template <int DT>
 struct Mfma;
+// run(): the compiler picks the registers.  run_agpr(): the accumulator is
+// pinned to the AGPR half of the register file.  A wave that owns a whole
+// SIMD has 256 + 256 registers; a 128x128 wave tile needs 256 accumulators,
+// and left to itself the register allocator keeps shuffling them between the
+// two halves around every MFMA.
 template <>
 struct Mfma<IRIS_DTYPE_BF16> {
   using vec8 = bf16x8;
   __device__ static inline f32x16 run(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline void run_agpr(vec8 a, vec8 b, f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  __device__ static inline void first_agpr(vec8 a, vec8 b, f32x16& c) {  // c = a x b
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
   }
 };
 template <>
@@ -71,6 +83,12 @@ struct Mfma<IRIS_DTYPE_F16> {
   using vec8 = f16x8;
   __device__ static inline f32x16 run(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline void run_agpr(vec8 a, vec8 b, f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  __device__ static inline void first_agpr(vec8 a, vec8 b, f32x16& c) {  // c = a x b
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
   }
 };
 
@@ -89,6 +107,7 @@ struct GemmCfg {
   static constexpr int A_LOADS = CM * CPR / NT, B_LOADS = CN * CPR / NT;
   static constexpr int L = A_LOADS + B_LOADS;
   static constexpr int KSUB = BK / 16;
+  static constexpr bool AGPR_ACC = IM * IN * 16 > 128;  // accumulators pinned to AGPRs
   // wave-private epilogue scratch: 32 rows x TN 16-bit elements
   static constexpr int WS_PITCH = TN * 2;
   static constexpr int WS_BYTES = 32 * WS_PITCH;
@@ -100,10 +119,9 @@ struct GemmCfg {
   static_assert((CM * CPR) % NT == 0 && (CN * CPR) % NT == 0, "slab must split evenly over lanes");
   static_assert(A_LOADS >= 1 && B_LOADS >= 1, "too many waves for this slab");
   static_assert((S & (S - 1)) == 0 && S >= 1, "ring depth must be a power of two");
-  static_assert(!DMA || S >= 4, "the DMA ring needs a stage being refilled, read, landed and in flight");
-  static_assert(L * (S > 2 ? S - 2 : 0) <= 63, "vmcnt immediate");
+  static_assert(!DMA || S >= 2, "the DMA ring needs a stage being read and one in flight");
+  static_assert(L * (S - 1) <= 63, "vmcnt immediate");
   static_assert(KSUB % 2 == 0, "fragment double-buffering alternates per K-substep");
-  static_assert(RPB % (RP * CPR) == 0, "XOR term of a DMA block must depend on the lane only");
   static_assert(TN == 32 || TN == 64 || TN == 128, "wave tile width");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
@@ -158,7 +176,8 @@ template <class Cfg>
 struct Loader {
   __amdgpu_buffer_rsrc_t ra, rb;
   uint32_t voff[Cfg::L];  // byte offset of (row, logical chunk) at k0 == 0
-  int kcol;               // first k of this lane's chunk at k0 == 0 (the same for every load)
+  int kcol[Cfg::L];       // first k of the chunk at k0 == 0
+  int k_limit;            // K, or 0 once the program has no more steps to load
 
   __device__ inline void setup(const GemmKArgs& p, const Item& it, int wave, int lane) {
     // Rows past the matrix edge re-read the last valid row (the reference
@@ -171,35 +190,41 @@ struct Loader {
     const uint32_t brec = (uint32_t)(((int64_t)(rows_b - 1) * p.sbn + p.K) * 2);
     ra = __builtin_amdgcn_make_buffer_rsrc((void*)abase, 0, arec, 0x00020000);
     rb = __builtin_amdgcn_make_buffer_rsrc((void*)bbase, 0, brec, 0x00020000);
-    // a 1 KiB block holds RPB = RP*CPR*k rows, so the row's XOR term depends
-    // on the lane only
-    const int ch = (lane % Cfg::CPR) ^ (((lane / Cfg::CPR) / Cfg::RP) % Cfg::CPR);
-    kcol = ch * 8;
+    k_limit = (p.debug & 1) ? 0 : p.K;
 #pragma unroll
     for (int i = 0; i < Cfg::L; ++i) {
       const bool isA = i < Cfg::A_LOADS;
       const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
       const int row = blk * Cfg::RPB + lane / Cfg::CPR;
+      const int ch = (lane % Cfg::CPR) ^ ((row / Cfg::RP) % Cfg::CPR);
       const int rclamp = min(row, (isA ? rows_a : rows_b) - 1);
       const int64_t ld = isA ? p.sam : p.sbn;
       voff[i] = (uint32_t)(((int64_t)rclamp * ld + ch * 8) * 2);
+      kcol[i] = ch * 8;
+      if (p.debug & 2) voff[i] = (uint32_t)(ch * 16);
     }
   }
 
-  // Issue the L loads of K-step `k` into the stage at LDS address `stage`.
-  __device__ inline void issue(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
+  // Issue load `i` of K-step `k` into the stage at LDS address `stage`.
+  // The K offset rides in the scalar offset; chunks past K read as zero: a
+  // vector offset beyond num_records is out of range for the buffer and the
+  // load returns 0 (the masked tail of gemm_*:186-195).  After the program's
+  // last step k_limit is 0: the loads are still issued, so that every K-step
+  // keeps the same number of loads in flight, but fetch nothing.
+  template <int I>
+  __device__ inline void issue_one(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
+    constexpr bool isA = I < Cfg::A_LOADS;
     const int k0 = k * Cfg::BK;
-    // chunks past K read as zero: an offset beyond num_records is out of
-    // range for the buffer and the load returns 0 (the masked tail of
-    // gemm_*:186-195)
-    const bool in_k = k0 + kcol < p.K;
-#pragma unroll
-    for (int i = 0; i < Cfg::L; ++i) {
-      const bool isA = i < Cfg::A_LOADS;
-      const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
-      IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + blk * 1024;
-      const uint32_t off = in_k ? voff[i] + (uint32_t)k0 * 2 : 0x80000000u;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, 0, 0, 0);
+    const int blk = (isA ? I : I - Cfg::A_LOADS) * Cfg::NW + wave;
+    IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + blk * 1024;
+    const uint32_t off = (k0 + kcol[I] < k_limit) ? voff[I] : 0x80000000u;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, k0 * 2, 0, 0);
+  }
+  template <int I = 0>
+  __device__ inline void issue(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
+    if constexpr (I < Cfg::L) {
+      issue_one<I>(p, stage, k, wave);
+      issue<I + 1>(p, stage, k, wave);
     }
   }
 };
@@ -251,33 +276,68 @@ struct Frags {
   typename Mfma<Cfg::DT>::vec8 a[Cfg::IM], b[Cfg::IN];
 };
 
-// Fetch the operand fragments of one K-substep (16 k) of a stage.
-template <class Cfg>
-__device__ inline void load_frags(const IRIS_LDS char* stage, int a_row_off, int b_row_off, int xo, Frags<Cfg>& f) {
+// Operand fragment F of one K-substep (16 k) of a stage: the B blocks first,
+// then the A blocks.  sA / sB point at this lane's row and chunk.
+template <class Cfg, int F>
+__device__ inline void load_frag(const IRIS_LDS char* sA, const IRIS_LDS char* sB, Frags<Cfg>& f) {
   using V = typename Mfma<Cfg::DT>::vec8;
-  const IRIS_LDS char* sA = stage + a_row_off + xo;
-  const IRIS_LDS char* sB = stage + Cfg::A_BYTES + b_row_off + xo;
-#pragma unroll
-  for (int j = 0; j < Cfg::IN; ++j) f.b[j] = *reinterpret_cast<const IRIS_LDS V*>(sB + j * 32 * Cfg::BK * 2);
-#pragma unroll
-  for (int i = 0; i < Cfg::IM; ++i) f.a[i] = *reinterpret_cast<const IRIS_LDS V*>(sA + i * 32 * Cfg::BK * 2);
+  if constexpr (F < Cfg::IN)
+    f.b[F] = *reinterpret_cast<const IRIS_LDS V*>(sB + F * 32 * Cfg::BK * 2);
+  else
+    f.a[F - Cfg::IN] = *reinterpret_cast<const IRIS_LDS V*>(sA + (F - Cfg::IN) * 32 * Cfg::BK * 2);
+}
+template <class Cfg, int F0, int F1>
+__device__ inline void load_frag_range(const IRIS_LDS char* sA, const IRIS_LDS char* sB, Frags<Cfg>& f) {
+  if constexpr (F0 < F1 && F0 < Cfg::IM + Cfg::IN) {
+    load_frag<Cfg, F0>(sA, sB, f);
+    load_frag_range<Cfg, F0 + 1, F1>(sA, sB, f);
+  }
 }
 
-// acc (+)= B-fragment x A-fragment for every 32x32 block of the wave tile.
-// FIRST starts a tile: the accumulator input is the constant 0.
-template <class Cfg, bool FIRST>
-__device__ inline void mma_frags(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& f) {
-#pragma unroll
-  for (int i = 0; i < Cfg::IM; ++i)
-#pragma unroll
-    for (int j = 0; j < Cfg::IN; ++j) {
-      if (FIRST) {
-        const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        acc[i][j] = Mfma<Cfg::DT>::run(f.b[j], f.a[i], z);
-      } else {
-        acc[i][j] = Mfma<Cfg::DT>::run(f.b[j], f.a[i], acc[i][j]);
-      }
+// acc (+)= B-fragment x A-fragment for 32x32 block BLK of the wave tile.
+// FIRST: the block's first product of a tile, which defines the accumulator.
+template <class Cfg, int BLK, bool FIRST = false>
+__device__ inline void mma_block(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& f) {
+  constexpr int i = BLK / Cfg::IN, j = BLK % Cfg::IN;
+  if constexpr (Cfg::AGPR_ACC) {
+    if constexpr (FIRST)
+      Mfma<Cfg::DT>::first_agpr(f.b[j], f.a[i], acc[i][j]);
+    else
+      Mfma<Cfg::DT>::run_agpr(f.b[j], f.a[i], acc[i][j]);
+  } else {
+    if constexpr (FIRST) {
+      const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+      acc[i][j] = Mfma<Cfg::DT>::run(f.b[j], f.a[i], z);
+    } else {
+      acc[i][j] = Mfma<Cfg::DT>::run(f.b[j], f.a[i], acc[i][j]);
     }
+  }
+}
+
+// Whole K-substep at once (used by the generic-loader path).
+template <class Cfg, bool FIRST, int BLK = 0>
+__device__ inline void mma_all(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& f) {
+  if constexpr (BLK < Cfg::IM * Cfg::IN) {
+    mma_block<Cfg, BLK, FIRST>(acc, f);
+    mma_all<Cfg, FIRST, BLK + 1>(acc, f);
+  }
+}
+
+// First half of a K-step: multiply substep `cur` while fetching the next
+// substep of the same stage.  Two fetches go out before the first MFMA, then
+// one per MFMA, so that every fetch has several MFMAs to land behind.
+template <class Cfg, bool FIRST, int BLK = 0>
+__device__ inline void mma_fetch_interleaved(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& cur,
+                                             const IRIS_LDS char* sA, const IRIS_LDS char* sB, Frags<Cfg>& nxt) {
+  constexpr int NB = Cfg::IM * Cfg::IN, NF = Cfg::IM + Cfg::IN;
+  if constexpr (BLK < NB) {
+    constexpr int F0 = BLK == 0 ? 0 : BLK + 1;
+    constexpr int F1 = BLK == NB - 1 ? NF : BLK + 2;  // the last block takes what is left
+    load_frag_range<Cfg, F0, F1>(sA, sB, nxt);
+    mma_block<Cfg, BLK, FIRST>(acc, cur);
+    __builtin_amdgcn_sched_barrier(0);
+    mma_fetch_interleaved<Cfg, FIRST, BLK + 1>(acc, cur, sA, sB, nxt);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -331,13 +391,17 @@ __device__ inline void atomic_add16_pair(IRIS_GLOBAL unsigned int* p, unsigned i
 // OP_ATOMIC32: fp32 atomic add                    OP_ATOMIC16: 16-bit atomic add
 template <class Cfg, int OP, int ODT>
 __device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM][Cfg::IN], IRIS_LDS char* ws,
-                                 int wm0, int wn0, int m_end, int n_end, int lane) {
+                                 int wm0, int wn0, int m_end, int n_end, int lane) {  // lane: by value, see below
   constexpr bool F32 = (OP == OP_STORE32 || OP == OP_ATOMIC32);
   constexpr int ES = F32 ? 4 : 2;
   constexpr int CP = Cfg::WS_PITCH / ES;  // columns per pass
   constexpr int NPASS = Cfg::TN / CP;     // 1 (16-bit) or 2 (fp32)
   constexpr int NQ = CP / 8;              // 8-column groups per pass
   constexpr int EPV = 16 / ES;            // elements per 16-byte unit
+  // Everything below depends on the lane id.  It is made opaque here so that
+  // the address arithmetic of the epilogue is computed in the epilogue and
+  // not hoisted into registers that stay live across the K loop.
+  asm volatile("" : "+v"(lane));
   const int lrow = lane & 31, lhalf = lane >> 5;
   const int r_begin = p.dest_all ? 0 : p.cur_rank;
   const int r_end = p.dest_all ? p.ws : p.cur_rank + 1;
@@ -466,6 +530,50 @@ __device__ inline void publish_tile(const GemmKArgs& p, int tile_id) {
   }
 }
 
+// Hand-over helpers of the last K-substep.  MFMA blocks 0 and 1 have been
+// issued before the barrier; the rest are issued here with, between them,
+// PER fragment fetches of the next stage each ...
+template <class Cfg, int BLK, int F = 0, int PER = 2>
+__device__ inline void hand_over_fetch_impl(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& cur,
+                                            const IRIS_LDS char* sA, const IRIS_LDS char* sB, Frags<Cfg>& nxt) {
+  constexpr int NB = Cfg::IM * Cfg::IN, NF = Cfg::IM + Cfg::IN;
+  if constexpr (F < NF) {
+    load_frag_range<Cfg, F, F + PER>(sA, sB, nxt);
+    if constexpr (BLK < NB) mma_block<Cfg, BLK>(acc, cur);
+    __builtin_amdgcn_sched_barrier(0);
+    hand_over_fetch_impl<Cfg, BLK + 1, F + PER, PER>(acc, cur, sA, sB, nxt);
+  }
+}
+template <class Cfg, int BLK>
+__device__ inline void hand_over_fetch(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& cur,
+                                       const IRIS_LDS char* sA, const IRIS_LDS char* sB, Frags<Cfg>& nxt) {
+  hand_over_fetch_impl<Cfg, BLK, 0, 2>(acc, cur, sA, sB, nxt);
+}
+
+// ... then one DMA load of the refilled stage per MFMA, then the MFMAs left.
+template <class Cfg, int BLK, int I = 0>
+__device__ inline void hand_over_dma(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& cur, const Loader<Cfg>& ld,
+                                     const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) {
+  constexpr int NB = Cfg::IM * Cfg::IN;
+  if constexpr (I < Cfg::L) {
+    ld.template issue_one<I>(p, stage, k, wave);
+    if constexpr (BLK < NB) mma_block<Cfg, BLK>(acc, cur);
+    __builtin_amdgcn_sched_barrier(0);
+    hand_over_dma<Cfg, BLK + 1, I + 1>(acc, cur, ld, p, stage, k, wave);
+  } else if constexpr (BLK < NB) {
+    mma_block<Cfg, BLK>(acc, cur);
+    hand_over_dma<Cfg, BLK + 1, I>(acc, cur, ld, p, stage, k, wave);
+  }
+}
+
+template <class Cfg, int BLK>
+__device__ inline void mma_rest(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& cur) {
+  if constexpr (BLK < Cfg::IM * Cfg::IN) {
+    mma_block<Cfg, BLK>(acc, cur);
+    mma_rest<Cfg, BLK + 1>(acc, cur);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // The kernel
 // ---------------------------------------------------------------------------
@@ -511,17 +619,22 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArg
   const bool defer_publish = Cfg::DMA && nk > 0 && p.flag_mode != 0;
   int pending_tile = -1;
 
-  int c_item = 0, c_k = 0;  // compute cursor
+  int c_item = 0;  // compute cursor
   Item c_it;
   if (n_items > 0) c_it = decode_item<Cfg>(p, pid, 0);
 
   // end of a compute tile: store it, and publish the logical tile it completes
   auto epilogue = [&]() __attribute__((always_inline)) {
+    if constexpr (Cfg::AGPR_ACC) {
+      // the compiler cannot see the latency of MFMAs issued from inline asm:
+      // let the last one (16 passes at most) retire before its result is read
+      asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15");
+    }
     store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end, c_it.n_end,
                             lane);
     if (c_it.last_sub) {
       if (defer_publish) {
-        pending_tile = c_it.tile_id;
+        pending_tile = __builtin_amdgcn_readfirstlane(c_it.tile_id);
       } else if (p.flag_mode != 0) {
         IRIS_WAIT_VMCNT(0);  // this wave's stores of the tile have completed
         __syncthreads();
@@ -543,108 +656,132 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArg
     // K == 0 leaves every tile all zeros: one epilogue per item, no loads
     for (int it = 0; it < n_items; ++it) epilogue();
   } else if constexpr (Cfg::DMA) {
-    // ---- the flattened (item, k) pipeline -------------------------------
-    // Ring of S stages.  While step g is multiplied: stage g is being read,
-    // stage g+1 has landed, stage g+2 is in flight and stage g-1 is being
-    // refilled with step g+3.
+    // ---- the (item, k) pipeline -------------------------------------------
+    // Ring of S stages.  A step's last fragment fetch happens one substep
+    // before its last MFMAs, so at the hand-over in step g every wave is done
+    // reading stage g: it is refilled right there with step g+S.  While the
+    // tail of step g is multiplied, stage g+1 has landed and stages
+    // g+2..g+S are in flight.  The load cursor runs S steps ahead of the
+    // compute cursor and crosses into the next item on its own.
     Loader<Cfg> ld;
     int l_item = 0, l_k = 0;  // load cursor
     Item l_it;
-    auto issue_next = [&](IRIS_LDS char* stage) __attribute__((always_inline)) {
-      ld.issue(p, stage, l_k, wave);
+    auto advance_load_cursor = [&]() __attribute__((always_inline)) {
       if (++l_k == nk) {
         l_k = 0;
         if (++l_item < n_items) {
           l_it = decode_item<Cfg>(p, pid, l_item);
           ld.setup(p, l_it, wave, lane);
+        } else {
+          ld.k_limit = 0;  // nothing left to load
         }
       }
     };
+    Frags<Cfg> fr[2];
+    constexpr int NB = Cfg::IM * Cfg::IN, NF = Cfg::IM + Cfg::IN;
     if (total_steps > 0) {
       l_it = decode_item<Cfg>(p, pid, 0);
       ld.setup(p, l_it, wave, lane);
 #pragma unroll
-      for (int s = 0; s < Cfg::S - 1; ++s)
-        if (s < total_steps) issue_next(lds + s * Cfg::STAGE);
-      // stage 0 has landed once at most S-2 younger slabs are outstanding
-      if (total_steps >= Cfg::S - 1) {
-        IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
-      } else {
-        IRIS_WAIT_VMCNT(0);
+      for (int s = 0; s < Cfg::S; ++s) {
+        ld.issue(p, lds + s * Cfg::STAGE, l_k, wave);
+        advance_load_cursor();
       }
+      // stage 0 has landed once at most S-1 younger slabs are outstanding
+      IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 1));
       block_barrier_raw();
+      load_frag_range<Cfg, 0, NF>(lds + a_row_off + xoff[0], lds + Cfg::A_BYTES + b_row_off + xoff[0], fr[0]);
+      IRIS_WAIT_LGKMCNT0();
     }
-    Frags<Cfg> fr[2];
-    if (total_steps > 0) load_frags<Cfg>(lds, a_row_off, b_row_off, xoff[0], fr[0]);
 
-    // One K-step.  LAST is the final step of the program: nothing is handed
-    // over or prefetched after it (kept out of the loop so that the loop body
-    // is straight-line code around its MFMAs).
-    auto step = [&](int g, auto last_tag) __attribute__((always_inline)) {
-      constexpr bool LAST = decltype(last_tag)::value;
+    // One K-step (global step number g).  FIRST: the tile's first step, whose
+    // first substep defines the accumulators.
+    //
+    // The step's MFMAs are issued in a fixed order with everything else
+    // slotted between them, so that the matrix cores always have work queued
+    // while the wave does its bookkeeping:
+    //   substeps 0..KSUB-2:  F F M F M F M ... M          (F: fragment fetch of the next substep)
+    //   last substep:        M M | wait, barrier | F F M F F M ... D M D M ... M
+    //                        (F: fetches from stage g+1, D: DMA loads of step g+S)
+    // The program's very last step hands over too; what it fetches and loads
+    // is never used (loads past the last step fetch nothing).
+    auto step = [&](int g, auto first_tag) __attribute__((always_inline)) {
+      constexpr bool FIRST = decltype(first_tag)::value;
       const IRIS_LDS char* stage = lds + (g & (Cfg::S - 1)) * Cfg::STAGE;
-      if (c_k == 0) stamp_begin();
 #pragma unroll
-      for (int kk = 0; kk < Cfg::KSUB; ++kk) {
-        // fetch the next K-substep's fragments before multiplying this one
-        if (kk + 1 < Cfg::KSUB) {
-          load_frags<Cfg>(stage, a_row_off, b_row_off, xoff[kk + 1], fr[(kk + 1) & 1]);
-        } else if (!LAST) {
-          // hand-over of stage g+1: wait for this wave's part of its slab
-          // (S-3 younger slabs may stay in flight), then meet the other waves
-          if (pending_tile >= 0 || g + Cfg::S - 2 > total_steps - 1) {
-            IRIS_WAIT_VMCNT(0);
-          } else {
-            IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 3));
-          }
-          block_barrier_raw();
-          if (pending_tile >= 0) {
-            if (tid == 0) publish_tile(p, pending_tile);
-            pending_tile = -1;
-          }
-          // every wave is past its reads of stage g-1: refill it
-          if (g + Cfg::S - 1 < total_steps) issue_next(lds + ((g + Cfg::S - 1) & (Cfg::S - 1)) * Cfg::STAGE);
-          load_frags<Cfg>(lds + ((g + 1) & (Cfg::S - 1)) * Cfg::STAGE, a_row_off, b_row_off, xoff[0], fr[0]);
-        }
-        __builtin_amdgcn_sched_barrier(0);  // fetches stay ahead of the MFMAs they overlap
-        if (kk == 0 && c_k == 0)
-          mma_frags<Cfg, true>(acc, fr[0]);
+      for (int kk = 0; kk < Cfg::KSUB - 1; ++kk) {
+        const IRIS_LDS char* sA = stage + a_row_off + xoff[kk + 1];
+        const IRIS_LDS char* sB = stage + Cfg::A_BYTES + b_row_off + xoff[kk + 1];
+        if (FIRST && kk == 0)
+          mma_fetch_interleaved<Cfg, true>(acc, fr[kk & 1], sA, sB, fr[(kk + 1) & 1]);
         else
-          mma_frags<Cfg, false>(acc, fr[kk & 1]);
-        // The fragments requested above have had this whole MFMA block to
-        // arrive.  Waiting for them here costs nothing and spares the next
-        // block a wait that would also cover the requests issued just before it.
-        __builtin_amdgcn_sched_barrier(0);
+          mma_fetch_interleaved<Cfg, false>(acc, fr[kk & 1], sA, sB, fr[(kk + 1) & 1]);
+        // the fetches above have had the MFMA block to arrive: waiting here is
+        // free and spares the next block a wait that would cover later requests
         IRIS_WAIT_LGKMCNT0();
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (++c_k == nk) {
-        c_k = 0;
-        epilogue();
+      {
+        constexpr int kk = Cfg::KSUB - 1;
+        const Frags<Cfg>& cur = fr[kk & 1];
+        // two MFMAs go out ahead of the hand-over
+        mma_block<Cfg, 0>(acc, cur);
+        if constexpr (NB > 1) mma_block<Cfg, 1>(acc, cur);
+        __builtin_amdgcn_sched_barrier(0);
+        // hand-over of stage g+1: wait for this wave's part of its slab
+        // (S-2 younger slabs may stay in flight), then meet the other waves
+        const int pend = __builtin_amdgcn_readfirstlane(pending_tile);
+        if (pend >= 0) {
+          IRIS_WAIT_VMCNT(0);  // the previous tile's stores, too
+        } else {
+          IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
+        }
+        block_barrier_raw();
+        if (pend >= 0) {
+          if (tid == 0) publish_tile(p, pend);
+          pending_tile = -1;
+        }
+        const IRIS_LDS char* nstage = lds + ((g + 1) & (Cfg::S - 1)) * Cfg::STAGE;
+        // fragment fetches of (g+1, substep 0), two per MFMA
+        hand_over_fetch<Cfg, 2>(acc, cur, nstage + a_row_off + xoff[0], nstage + Cfg::A_BYTES + b_row_off + xoff[0],
+                                fr[0]);
+        // every wave is past its reads of stage g: refill it, one load per MFMA
+        IRIS_LDS char* rstage = lds + (g & (Cfg::S - 1)) * Cfg::STAGE;
+        hand_over_dma<Cfg, 2 + (NF + 1) / 2>(acc, cur, ld, p, rstage, l_k, wave);
+        advance_load_cursor();
+        IRIS_WAIT_LGKMCNT0();
+        __builtin_amdgcn_sched_barrier(0);
       }
     };
-    for (int g = 0; g < total_steps - 1; ++g) step(g, std::false_type{});
-    if (total_steps > 0) step(total_steps - 1, std::true_type{});
+    int g = 0;
+    for (int it = 0; it < n_items; ++it) {
+      stamp_begin();
+      step(g, std::true_type{});
+      ++g;
+      for (int k = 1; k < nk; ++k, ++g) step(g, std::false_type{});
+      epilogue();
+    }
+    IRIS_WAIT_VMCNT(0);  // no load may still be writing this group's LDS when it exits
   } else {
     // ---- generic loader: one stage, synchronous ---------------------------
     Frags<Cfg> fr;
-    for (int g = 0; g < total_steps; ++g) {
-      __syncthreads();  // previous step's readers are done with the stage
-      load_slab_generic<Cfg>(p, c_it, lds, c_k, tid);
-      __syncthreads();
-      if (c_k == 0) stamp_begin();
+    for (int it = 0; it < n_items; ++it) {
+      stamp_begin();
+      for (int k = 0; k < nk; ++k) {
+        __syncthreads();  // previous step's readers are done with the stage
+        load_slab_generic<Cfg>(p, c_it, lds, k, tid);
+        __syncthreads();
 #pragma unroll
-      for (int kk = 0; kk < Cfg::KSUB; ++kk) {
-        load_frags<Cfg>(lds, a_row_off, b_row_off, xoff[kk], fr);
-        if (kk == 0 && c_k == 0)
-          mma_frags<Cfg, true>(acc, fr);
-        else
-          mma_frags<Cfg, false>(acc, fr);
+        for (int kk = 0; kk < Cfg::KSUB; ++kk) {
+          load_frag_range<Cfg, 0, Cfg::IM + Cfg::IN>(lds + a_row_off + xoff[kk],
+                                                     lds + Cfg::A_BYTES + b_row_off + xoff[kk], fr);
+          if (k == 0 && kk == 0)
+            mma_all<Cfg, true>(acc, fr);
+          else
+            mma_all<Cfg, false>(acc, fr);
+        }
       }
-      if (++c_k == nk) {
-        c_k = 0;
-        epilogue();
-      }
+      epilogue();
     }
   }
 

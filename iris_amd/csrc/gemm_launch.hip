@@ -132,6 +132,10 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   k.total_tiles = k.num_pid_m * k.num_pid_n;
   k.sys = a.scope == IRIS_SCOPE_SYSTEM;
   k.vec_out = vec_ok(k.out, k.som, k.son, dtype_size(out_dt)) ? 1 : 0;
+  {
+    static const int dbgflags = std::getenv("IRIS_AMD_GEMM_DEBUG") ? std::atoi(std::getenv("IRIS_AMD_GEMM_DEBUG")) : 0;
+    k.debug = dbgflags;
+  }
 
   int count = 0;
   const GemmKernelEntry* list = entries_for(a.ab_dtype, op, &count);

@@ -33,7 +33,7 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 // compute tile divides the logical tile (and whose loader fits the operands)
 // wins.  `variant` k > 0 in iris_gemm_args forces entry k-1 (tuning runs).
 #define IRIS_GEMM_VARIANTS(X, DT, OP)                            \
-  X(DT, OP, 256, 256, 32, 2, 4, 4, true, "256x256x32_w2x4_s4")   \
+  X(DT, OP, 256, 256, 64, 2, 4, 2, true, "256x256x64_w2x4_s2")   \
   X(DT, OP, 256, 128, 32, 2, 2, 4, true, "256x128x32_w2x2_s4")   \
   X(DT, OP, 128, 256, 32, 2, 2, 4, true, "128x256x32_w2x2_s4")   \
   X(DT, OP, 128, 128, 32, 2, 2, 4, true, "128x128x32_w2x2_s4")   \
@@ -44,8 +44,11 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 // extra variants of the headline tile, compiled for the bf16 store op only
 #define IRIS_GEMM_TUNING_VARIANTS(X, DT, OP)                     \
   X(DT, OP, 256, 256, 32, 2, 2, 4, true, "256x256x32_w2x2_s4")   \
+  X(DT, OP, 256, 256, 64, 2, 2, 2, true, "256x256x64_w2x2_s2")   \
+  X(DT, OP, 256, 256, 32, 2, 4, 4, true, "256x256x32_w2x4_s4")   \
   X(DT, OP, 256, 128, 32, 2, 4, 4, true, "256x128x32_w2x4_s4")   \
-  X(DT, OP, 128, 128, 32, 2, 2, 8, true, "128x128x32_w2x2_s8")
+  X(DT, OP, 256, 128, 64, 2, 4, 2, true, "256x128x64_w2x4_s2")   \
+  X(DT, OP, 256, 128, 64, 2, 2, 2, true, "256x128x64_w2x2_s2")
 
 #define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, NAME) \
   make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP>(NAME),

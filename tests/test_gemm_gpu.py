@@ -188,12 +188,14 @@ def test_unaligned_and_strided_output(shmem):
     check_close(c32, O.shard_gemm(A, B, None))
 
 
-@pytest.mark.parametrize("variant", range(1, 11))
+@pytest.mark.parametrize("variant", range(1, 25))
 def test_every_tuning_variant_is_correct(shmem, variant):
     """Each compiled kernel variant of the bf16 store path, forced on a shape
     with ragged edges and several tiles per program."""
     name = ops.gemm_variant_name(torch.bfloat16, False, False, variant)
-    assert name is not None
+    if name is None:
+        assert variant > 7  # the seven base tiles always exist
+        pytest.skip("no such variant")
     dtype = torch.bfloat16
     M, N, K = 520, 776, 328
     A, B = make_ab(M, N, K, dtype, lda=336, ldb=344)
@@ -205,7 +207,6 @@ def test_every_tuning_variant_is_correct(shmem, variant):
     torch.cuda.synchronize()
     check_close(cg, O.shard_gemm(A, B, dtype), name)
     assert flags.cpu().tolist() == [1] * total
-    assert ops.gemm_variant_name(torch.bfloat16, False, False, 11) is None
 
 
 # --------------------------------------------------------------------------- atomics
