@@ -55,7 +55,7 @@ struct GemmKArgs {
   int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
   int sys;           // flag atomics at system scope (else agent)
   int vec_out;       // 16-byte vector access allowed on `out`
-  int debug;         // tuning experiments only (IRIS_AMD_GEMM_DEBUG): 1 = fetch nothing, 2 = every row fetches row 0
+  int debug;         // tuning experiments only (IRIS_AMD_GEMM_DEBUG): 1 = fetch nothing, 2 = every row fetches row 0, 4 = store nothing
 };
 
 template <int DT>
@@ -630,8 +630,9 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArg
       // let the last one (16 passes at most) retire before its result is read
       asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15");
     }
-    store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end, c_it.n_end,
-                            lane);
+    if (!(p.debug & 4))
+      store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end, c_it.n_end,
+                              lane);
     if (c_it.last_sub) {
       if (defer_publish) {
         pending_tile = __builtin_amdgcn_readfirstlane(c_it.tile_id);

@@ -5,9 +5,9 @@
 // the tile over ranks 0..ws-1 in fp32 and store it to c_global.
 //
 // The kernel is HBM-bound: per output element it reads ws partials and writes
-// one result.  Each lane moves 8 consecutive columns per step (two 16-byte
-// loads per rank for fp32 partials), lanes run along a row so that a wave
-// covers whole contiguous row segments, and several steps are kept in flight.
+// one result.  Each lane moves one 16-byte strip per rank and step, lanes run
+// along a row so that a wave covers contiguous row segments, and the strips
+// of several rows are kept in flight.
 #pragma once
 
 #include "common.hpp"
@@ -29,43 +29,56 @@ struct ReduceKArgs {
   int sys, wait_flags;
 };
 
+// VE<DT>: elements in one 16-byte load of type DT.  A lane always moves 16
+// bytes per rank, so that one wave-wide load covers 1 KiB of contiguous
+// memory; wider per-lane strips (two loads a lane) measured ~20% slower.
+template <int DT>
+struct Vec {
+  static constexpr int ES = (DT == IRIS_DTYPE_F32) ? 4 : 2;
+  static constexpr int N = 16 / ES;
+};
+
+// Loads and stores go through buffer descriptors that span exactly one tile:
+// the hardware bounds check returns zeros for (and drops stores of) strips
+// below a ragged tile's last row, so the inner loop has no branches, and a
+// lane that owns no strip parks its offset at DEAD_OFFSET.
+constexpr uint32_t DEAD_OFFSET = 0x80000000u;
+constexpr int AUX_NT = 2;  // nontemporal bit of the buffer instructions' cache policy
+
+__device__ inline __amdgpu_buffer_rsrc_t tile_rsrc(const IRIS_GLOBAL char* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
+}
+
 template <int DT, bool NT>
-__device__ inline void load8(const IRIS_GLOBAL char* p, float (&v)[8]) {
+__device__ inline void load_vec(__amdgpu_buffer_rsrc_t rs, uint32_t off, float (&v)[Vec<DT>::N]) {
+  const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, NT ? AUX_NT : 0);
   if constexpr (DT == IRIS_DTYPE_F32) {
-    const IRIS_GLOBAL f32x4* q = reinterpret_cast<const IRIS_GLOBAL f32x4*>(p);
-    const f32x4 x0 = NT ? __builtin_nontemporal_load(q) : q[0];
-    const f32x4 x1 = NT ? __builtin_nontemporal_load(q + 1) : q[1];
+    // cast the whole vector: a bit_cast of one element reads element 0
+    const f32x4 f = __builtin_bit_cast(f32x4, x);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      v[e] = x0[e];
-      v[4 + e] = x1[e];
-    }
+    for (int e = 0; e < 4; ++e) v[e] = f[e];
   } else {
-    const IRIS_GLOBAL u32x4* q = reinterpret_cast<const IRIS_GLOBAL u32x4*>(p);
-    const u32x4 x = NT ? __builtin_nontemporal_load(q) : q[0];
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = from16<DT>((unsigned short)(x[e / 2] >> (16 * (e & 1))));
   }
 }
 
-template <int DT, bool NT>
-__device__ inline void store8(IRIS_GLOBAL char* p, const float (&v)[8]) {
+// store NE fp32 values as elements of type DT
+template <int DT, int NE, bool NT>
+__device__ inline void store_vec(__amdgpu_buffer_rsrc_t rs, uint32_t off, const float (&v)[NE]) {
+  constexpr int aux = NT ? AUX_NT : 0;
   if constexpr (DT == IRIS_DTYPE_F32) {
-    IRIS_GLOBAL f32x4* q = reinterpret_cast<IRIS_GLOBAL f32x4*>(p);
-    const f32x4 y0 = {v[0], v[1], v[2], v[3]}, y1 = {v[4], v[5], v[6], v[7]};
-    if (NT) {
-      __builtin_nontemporal_store(y0, q);
-      __builtin_nontemporal_store(y1, q + 1);
-    } else {
-      q[0] = y0;
-      q[1] = y1;
+#pragma unroll
+    for (int h = 0; h < NE / 4; ++h) {
+      const f32x4 f = {v[4 * h], v[4 * h + 1], v[4 * h + 2], v[4 * h + 3]};
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, f), rs, (int)(off + 16 * h), 0, aux);
     }
+  } else if constexpr (NE == 4) {
+    const u32x2 y = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+    __builtin_amdgcn_raw_buffer_store_b64(y, rs, (int)off, 0, aux);
   } else {
     const u32x4 y = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3]), pack2<DT>(v[4], v[5]), pack2<DT>(v[6], v[7])};
-    if (NT)
-      __builtin_nontemporal_store(y, reinterpret_cast<IRIS_GLOBAL u32x4*>(p));
-    else
-      *reinterpret_cast<IRIS_GLOBAL u32x4*>(p) = y;
+    __builtin_amdgcn_raw_buffer_store_b128(y, rs, (int)off, 0, aux);
   }
 }
 
@@ -86,75 +99,84 @@ __device__ inline bool block_wait_tile(const ReduceKArgs& p, int tile_id, IRIS_L
 }
 
 // Vector kernel: unit-stride columns, 16-byte aligned rows, tile widths that
-// are multiples of 8.  WS > 0 fixes the rank count at compile time.
+// are multiples of the vector width.  WS > 0 fixes the rank count at compile
+// time.  A lane owns one 16-byte strip per rank; UNROLL rows of the tile are
+// in flight per lane, i.e. WS * UNROLL independent loads.
 template <int IN_DT, int OUT_DT, int WS, int UNROLL, bool NT>
 __global__ __launch_bounds__(256) void reduce_tiles_vec_kernel(const ReduceKArgs p) {
   __shared__ int slot;
   const int ws = WS > 0 ? WS : p.ws;
-  constexpr int IES = (IN_DT == IRIS_DTYPE_F32) ? 4 : 2;
-  constexpr int OES = (OUT_DT == IRIS_DTYPE_F32) ? 4 : 2;
+  constexpr int IES = Vec<IN_DT>::ES, VE = Vec<IN_DT>::N;
+  constexpr int OES = Vec<OUT_DT>::ES;
   const int tid = threadIdx.x;
-  const uint64_t cur_base = p.heap_bases ? p.heap_bases[p.cur_rank] : 0;
+  const uint64_t cur_base = p.heap_bases ? uniform_u64(p.heap_bases[p.cur_rank]) : 0;
 
   for (int tile_id = xcd_remap(blockIdx.x, gridDim.x, p.num_xcds); tile_id < p.total_tiles; tile_id += gridDim.x) {
     const TileCoord tc = tile_map(tile_id, p.num_pid_m, p.num_pid_n, p.G);
     const int m0 = tc.pid_m * p.BM, n0 = tc.pid_n * p.BN;
     const int rows = min(p.M, m0 + p.BM) - m0, cols = min(p.N, n0 + p.BN) - n0;
     if (!block_wait_tile(p, tile_id, (IRIS_LDS int*)&slot)) continue;
-    const int c8 = cols / 8;
-    const int units = rows * c8;
-    IRIS_GLOBAL char* out0 = (IRIS_GLOBAL char*)p.cg + ((int64_t)m0 * p.sgm + n0) * OES;
+    const int cv = cols / VE;  // 16-byte strips per tile row
+    // Lanes run along a tile row; the block covers `rpp` rows per pass and
+    // UNROLL passes are in flight.
+    const int tpr = min(cv, 256), rpp = 256 / tpr;
+    const int r0 = tid / tpr, cl = tid - r0 * tpr;
+    const uint32_t in_bytes = ((uint32_t)(rows - 1) * (uint32_t)p.scm + cols) * IES;
+    const uint32_t out_bytes = ((uint32_t)(rows - 1) * (uint32_t)p.sgm + cols) * OES;
     const int64_t in0 = ((int64_t)m0 * p.scm + n0) * IES;
+    const __amdgpu_buffer_rsrc_t out_rs =
+        tile_rsrc((const IRIS_GLOBAL char*)p.cg + ((int64_t)m0 * p.sgm + n0) * OES, out_bytes);
+    auto rank_rsrc = [&](int rk) __attribute__((always_inline)) {
+      const IRIS_GLOBAL char* b = (rk == p.cur_rank || !p.heap_bases)
+                                      ? (const IRIS_GLOBAL char*)p.c
+                                      : translate(p.c, cur_base, uniform_u64(p.heap_bases[rk]));
+      return tile_rsrc(b + in0, in_bytes);
+    };
 
-    for (int u0 = tid; u0 < units; u0 += 256 * UNROLL) {
-      float acc[UNROLL][8];
-      int64_t ioff[UNROLL], ooff[UNROLL];
-      bool live[UNROLL];
+    for (int cc = 0; cc < cv; cc += tpr) {
+      const int c = cc + cl;
+      const bool col_live = r0 < rpp && c < cv;
+      for (int rb = 0; rb < rows; rb += rpp * UNROLL) {
+        float acc[UNROLL][VE];
+        uint32_t ioff[UNROLL], ooff[UNROLL];
 #pragma unroll
-      for (int s = 0; s < UNROLL; ++s) {
-        const int u = u0 + s * 256;
-        live[s] = u < units;
-        const int uu = live[s] ? u : 0;
-        const int r = uu / c8, c = (uu - r * c8) * 8;
-        ioff[s] = in0 + ((int64_t)r * p.scm + c) * IES;
-        ooff[s] = ((int64_t)r * p.sgm + c) * OES;
+        for (int s = 0; s < UNROLL; ++s) {
+          const uint32_t row = rb + r0 + s * rpp;
+          ioff[s] = col_live ? (row * (uint32_t)p.scm + c * VE) * IES : DEAD_OFFSET;
+          ooff[s] = col_live ? (row * (uint32_t)p.sgm + c * VE) * OES : DEAD_OFFSET;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[s][e] = 0.f;
-      }
-      // fixed rank order 0..ws-1 (gemm_one_shot_all_reduce.py:267-269)
-      if constexpr (WS > 0) {
-        float v[WS][UNROLL][8];
+          for (int e = 0; e < VE; ++e) acc[s][e] = 0.f;
+        }
+        // fixed rank order 0..ws-1 (gemm_one_shot_all_reduce.py:267-269)
+        if constexpr (WS > 0) {
+          float v[WS][UNROLL][VE];
 #pragma unroll
-        for (int rk = 0; rk < WS; ++rk) {
-          const IRIS_GLOBAL char* base = (rk == p.cur_rank || !p.heap_bases)
-                                             ? (const IRIS_GLOBAL char*)p.c
-                                             : translate(p.c, cur_base, p.heap_bases[rk]);
+          for (int rk = 0; rk < WS; ++rk) {
+            const __amdgpu_buffer_rsrc_t rs = rank_rsrc(rk);
 #pragma unroll
-          for (int s = 0; s < UNROLL; ++s) load8<IN_DT, NT>(base + ioff[s], v[rk][s]);
+            for (int s = 0; s < UNROLL; ++s) load_vec<IN_DT, NT>(rs, ioff[s], v[rk][s]);
+          }
+#pragma unroll
+          for (int rk = 0; rk < WS; ++rk)
+#pragma unroll
+            for (int s = 0; s < UNROLL; ++s)
+#pragma unroll
+              for (int e = 0; e < VE; ++e) acc[s][e] += v[rk][s][e];
+        } else {
+          for (int rk = 0; rk < ws; ++rk) {
+            const __amdgpu_buffer_rsrc_t rs = rank_rsrc(rk);
+            float v[UNROLL][VE];
+#pragma unroll
+            for (int s = 0; s < UNROLL; ++s) load_vec<IN_DT, NT>(rs, ioff[s], v[s]);
+#pragma unroll
+            for (int s = 0; s < UNROLL; ++s)
+#pragma unroll
+              for (int e = 0; e < VE; ++e) acc[s][e] += v[s][e];
+          }
         }
 #pragma unroll
-        for (int rk = 0; rk < WS; ++rk)
-#pragma unroll
-          for (int s = 0; s < UNROLL; ++s)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc[s][e] += v[rk][s][e];
-      } else {
-        for (int rk = 0; rk < ws; ++rk) {
-          const IRIS_GLOBAL char* base = (rk == p.cur_rank || !p.heap_bases)
-                                             ? (const IRIS_GLOBAL char*)p.c
-                                             : translate(p.c, cur_base, p.heap_bases[rk]);
-          float v[UNROLL][8];
-#pragma unroll
-          for (int s = 0; s < UNROLL; ++s) load8<IN_DT, NT>(base + ioff[s], v[s]);
-#pragma unroll
-          for (int s = 0; s < UNROLL; ++s)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc[s][e] += v[s][e];
-        }
+        for (int s = 0; s < UNROLL; ++s) store_vec<OUT_DT, VE, NT>(out_rs, ooff[s], acc[s]);
       }
-#pragma unroll
-      for (int s = 0; s < UNROLL; ++s)
-        if (live[s]) store8<OUT_DT, NT>(out0 + ooff[s], acc[s]);
     }
   }
 }

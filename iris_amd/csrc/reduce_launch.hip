@@ -22,7 +22,7 @@ ReduceFn pick_vec(int ws, int variant) {
       case 3: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 4, true>;
       case 4: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 1, false>;
       case 5: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 2, false>;
-      case 6: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 4, false>;
+      case 6: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 3, true>;
       default: return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 2, true>;
     }
   }
@@ -98,8 +98,13 @@ extern "C" int iris_one_shot_reduce_launch(const iris_reduce_args* a, void* stre
   k.num_xcds = (a->num_xcds > 1 && grid % a->num_xcds == 0) ? a->num_xcds : 1;
 
   const int ies = dtype_size(k.c_dt), oes = dtype_size(k.cg_dt);
+  // a lane moves 16 bytes of input at a time: 4 fp32 or 8 16-bit columns
+  const int ve = 16 / ies;
   const bool vec = k.scn == 1 && k.sgn == 1 && aligned16(k.c) && aligned16(k.cg) && (k.scm * ies) % 16 == 0 &&
-                   (k.sgm * oes) % 16 == 0 && k.BN % 8 == 0 && k.N % 8 == 0;
+                   (k.sgm * oes) % 16 == 0 && k.BN % ve == 0 && k.N % ve == 0 && (k.BN * oes) % 16 == 0 &&
+                   // lane offsets inside a tile are 32-bit
+                   k.scm >= k.N && k.sgm >= k.N && ((int64_t)k.BM + 256) * k.scm * ies < (1ll << 31) &&
+                   ((int64_t)k.BM + 256) * k.sgm * oes < (1ll << 31);
   ReduceFn fn = vec ? pick(k.c_dt, k.cg_dt, k.ws, a->variant) : nullptr;
   if (!fn) fn = &reduce_tiles_generic_kernel;
   hipLaunchKernelGGL(fn, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), k);
