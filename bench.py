@@ -28,6 +28,13 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E, published
 
+# HBM-side bytes per launch of the default kernels on this workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script, each scaled by what the same counter reads for the --copy-calibration
+# kernel (profiles/gemm_all_scatter_bf16_8192x8192x1024.txt, profiles/one_shot_reduce_fp32x8_8192x8192.txt).
+# Counters cannot be read from inside a run, so these are carried here and dropped for non-default variants.
+GEMM_TRAFFIC_BYTES = 332877946
+REDUCE_TRAFFIC_BYTES = 2281385094
+
 M, N, K_SHARD, K_TOTAL = 8192, 8192, 1024, 8192
 BLK_M, BLK_N, BLK_K, GSIZE_M, GRID = 256, 256, 64, 4, 256
 
@@ -35,8 +42,12 @@ BLK_M, BLK_N, BLK_K, GSIZE_M, GRID = 256, 256, 64, 4, 256
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="untimed launches of the same step before the warm-up, until this much time has passed: after "
+                         "an idle period the GPU's power management first overshoots and then clamps the clocks for "
+                         "~10 ms, which a short run would measure instead of the steady state")
     ap.add_argument("--variant", type=int, default=0, help="GEMM kernel tuning variant (0 = default)")
     ap.add_argument("--reduce-variant", type=int, default=0)
     ap.add_argument("--gsize_m", type=int, default=GSIZE_M)
@@ -44,29 +55,34 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-coldcache", action="store_true", help="skip the cold-cache do_bench protocol run")
     ap.add_argument("--offheap-operands", action="store_true", help="keep A and B outside the fine-grained heap")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a plain fp32 copy of [8192,8192] (256 MiB in, 256 MiB out): the kernel of known "
+                         "size that scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     return ap.parse_args()
 
 
 def timed_steps(fn, steps, warmup):
-    """(wall seconds for `steps` calls, mean per-call device ms from HIP events
-    recorded on the launch stream)."""
+    """(wall seconds for `steps` calls, mean per-launch device ms).
+
+    The device time comes from one pair of HIP events on the launch stream
+    around the `steps` back-to-back launches: an event between every two
+    launches would insert a ~11 us idle gap and a cache write-back before each
+    kernel, which is not how the path runs.
+    """
     import torch
 
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    for i in range(steps):
-        starts[i].record()
+    start.record()
+    for _ in range(steps):
         fn()
-        ends[i].record()
+    end.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    dev_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    return wall, dev_ms
+    return wall, start.elapsed_time(end) / steps
 
 
 def cpu_baseline():
@@ -88,7 +104,18 @@ def cpu_baseline():
         O.shard_gemm(A, B, torch.bfloat16)
         times.append(time.perf_counter() - t0)
     med = statistics.median(times)
+    # the reduce phase of the same math: 8 fp32 partials [1024, 8192] summed in rank order -> bf16
+    parts = torch.randn(8, 1024, N, generator=g)
+    O.one_shot_reduce(parts, torch.bfloat16)
+    rtimes = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        O.one_shot_reduce(parts, torch.bfloat16)
+        rtimes.append(time.perf_counter() - t0)
+    rmed = statistics.median(rtimes)
     return {
+        "reduce_GBps": round((parts.numel() * 4 + 1024 * N * 2) / rmed / 1e9, 2),
+        "reduce_sample": "oracle one_shot_reduce of 8 fp32 partials [1024,8192] -> bf16, 3 runs, median",
         "value": 2.0 * rows * N * K_SHARD / med / 1e12,
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
@@ -143,12 +170,18 @@ def main():
                         ops.EPI_ALL_SCATTER, notify=True, num_xcds=num_xcds, variant=args.variant)
 
     flops = 2.0 * M * N * K_SHARD
-    wall, dev_ms = timed_steps(gemm_step, args.steps, args.warmup)
+    settle_launches = 0
+    t_end = time.perf_counter() + args.settle_ms * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(20):
+            gemm_step()
+        torch.cuda.synchronize()
+        settle_launches += 20
+    wall, kernel_ms = timed_steps(gemm_step, args.steps, args.warmup)
     ms_per_step = wall / args.steps * 1e3
-    kernel_ms = statistics.mean(dev_ms)
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     kernel_tflops = flops / (kernel_ms * 1e-3) / 1e12
-    assert int(flags.min().item()) == args.steps + args.warmup, "every tile publishes once per step"
+    assert int(flags.min().item()) == args.steps + args.warmup + settle_launches, "every tile publishes once per step"
     regs, spills = ops.gemm_kernel_info(a, b, None, c_global, flags, hb, 0, 1, GRID, BLK_M, BLK_N, BLK_K,
                                         args.gsize_m, ops.EPI_ALL_SCATTER, num_xcds=num_xcds, variant=args.variant)
 
@@ -159,6 +192,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": args.settle_ms,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -174,15 +208,14 @@ def main():
             "operands": "device memory outside the heap" if args.offheap_operands else "fine-grained heap",
         },
         "pct_of_bf16_peak": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),
-        "gemm_kernel": {"registers": regs, "spill_bytes": spills, "mean_ms": round(kernel_ms, 5),
-                        "min_ms": round(min(dev_ms), 5)},
+        "gemm_kernel": {"registers": regs, "spill_bytes": spills, "mean_ms": round(kernel_ms, 5)},
         "roofline": {
             "bound": "mfma",
             "achieved": round(kernel_tflops, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(kernel_tflops / PEAK_BF16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES if args.variant == 0 and args.gsize_m == GSIZE_M else None,
         },
     }
 
@@ -226,8 +259,20 @@ def main():
             "mean_ms": round(rms, 5), "min_ms": round(min(red_ms), 5), "GBps": round(gbps, 1),
             "pct_of_hbm_peak": round(100.0 * gbps / PEAK_HBM_GBPS, 2), "variant": args.reduce_variant,
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                         "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": None},
+                         "frac": round(gbps / PEAK_HBM_GBPS, 4),
+                         "traffic": REDUCE_TRAFFIC_BYTES if args.reduce_variant == 0 else None},
         }
+
+    if args.copy_calibration:
+        # ws=1, fp32 -> fp32: the reduce kernel degenerates to a plain tiled copy
+        src = torch.randn((M, N), dtype=torch.float32, device="cuda")
+        dst = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        for _ in range(3):
+            ops.one_shot_reduce(src, dst, flags, hb, 0, 1, BLK_M, BLK_N, args.gsize_m, wait_flags=False)
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst)
+        result["copy_calibration"] = {"kernel": "reduce_tiles_vec_kernel<fp32, fp32, ws=1>",
+                                      "read_bytes": M * N * 4, "write_bytes": M * N * 4, "launches": 3}
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()

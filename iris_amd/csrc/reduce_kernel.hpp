@@ -43,15 +43,16 @@ struct Vec {
 // below a ragged tile's last row, so the inner loop has no branches, and a
 // lane that owns no strip parks its offset at DEAD_OFFSET.
 constexpr uint32_t DEAD_OFFSET = 0x80000000u;
-constexpr int AUX_NT = 2;  // nontemporal bit of the buffer instructions' cache policy
+// cache-policy bits of the buffer instructions
+constexpr int AUX_SC0 = 1, AUX_NT = 2, AUX_SC1 = 16;
 
 __device__ inline __amdgpu_buffer_rsrc_t tile_rsrc(const IRIS_GLOBAL char* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
 }
 
-template <int DT, bool NT>
+template <int DT, int AUX>
 __device__ inline void load_vec(__amdgpu_buffer_rsrc_t rs, uint32_t off, float (&v)[Vec<DT>::N]) {
-  const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, NT ? AUX_NT : 0);
+  const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, AUX);
   if constexpr (DT == IRIS_DTYPE_F32) {
     // cast the whole vector: a bit_cast of one element reads element 0
     const f32x4 f = __builtin_bit_cast(f32x4, x);
@@ -64,9 +65,9 @@ __device__ inline void load_vec(__amdgpu_buffer_rsrc_t rs, uint32_t off, float (
 }
 
 // store NE fp32 values as elements of type DT
-template <int DT, int NE, bool NT>
+template <int DT, int NE, int AUX>
 __device__ inline void store_vec(__amdgpu_buffer_rsrc_t rs, uint32_t off, const float (&v)[NE]) {
-  constexpr int aux = NT ? AUX_NT : 0;
+  constexpr int aux = AUX;
   if constexpr (DT == IRIS_DTYPE_F32) {
 #pragma unroll
     for (int h = 0; h < NE / 4; ++h) {
@@ -84,16 +85,19 @@ __device__ inline void store_vec(__amdgpu_buffer_rsrc_t rs, uint32_t off, const 
 
 // Block-wide wait for one tile's flag.  One lane polls; the outcome is
 // broadcast through LDS and every wave then acquires.
+template <bool FENCE = true>
 __device__ inline bool block_wait_tile(const ReduceKArgs& p, int tile_id, IRIS_LDS int* slot) {
   if (!p.wait_flags || p.ws <= 1) return true;
   if (threadIdx.x == 0)
     *slot = wait_tile_flag((IRIS_GLOBAL int32_t*)(p.flags + tile_id), p.ws, p.sys != 0, p.timeout, p.status) ? 1 : 0;
   __syncthreads();
   const int ok = *slot;
-  if (p.sys)
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-  else
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  if constexpr (FENCE) {
+    if (p.sys)
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+    else
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
   __syncthreads();  // the slot may be rewritten for the next tile
   return ok != 0;
 }
@@ -102,8 +106,11 @@ __device__ inline bool block_wait_tile(const ReduceKArgs& p, int tile_id, IRIS_L
 // are multiples of the vector width.  WS > 0 fixes the rank count at compile
 // time.  A lane owns one 16-byte strip per rank; UNROLL rows of the tile are
 // in flight per lane, i.e. WS * UNROLL independent loads.
-template <int IN_DT, int OUT_DT, int WS, int UNROLL, bool NT>
+template <int IN_DT, int OUT_DT, int WS, int UNROLL, int LAUX>
 __global__ __launch_bounds__(256) void reduce_tiles_vec_kernel(const ReduceKArgs p) {
+  // Loads that carry sc1 are coherent at the flags' scope by themselves: they
+  // never hit a stale line, so the wait needs no cache-invalidating fence.
+  constexpr bool FENCE = (LAUX & AUX_SC1) == 0;
   __shared__ int slot;
   const int ws = WS > 0 ? WS : p.ws;
   constexpr int IES = Vec<IN_DT>::ES, VE = Vec<IN_DT>::N;
@@ -115,7 +122,7 @@ __global__ __launch_bounds__(256) void reduce_tiles_vec_kernel(const ReduceKArgs
     const TileCoord tc = tile_map(tile_id, p.num_pid_m, p.num_pid_n, p.G);
     const int m0 = tc.pid_m * p.BM, n0 = tc.pid_n * p.BN;
     const int rows = min(p.M, m0 + p.BM) - m0, cols = min(p.N, n0 + p.BN) - n0;
-    if (!block_wait_tile(p, tile_id, (IRIS_LDS int*)&slot)) continue;
+    if (!block_wait_tile<FENCE>(p, tile_id, (IRIS_LDS int*)&slot)) continue;
     const int cv = cols / VE;  // 16-byte strips per tile row
     // Lanes run along a tile row; the block covers `rpp` rows per pass and
     // UNROLL passes are in flight.
@@ -154,7 +161,7 @@ __global__ __launch_bounds__(256) void reduce_tiles_vec_kernel(const ReduceKArgs
           for (int rk = 0; rk < WS; ++rk) {
             const __amdgpu_buffer_rsrc_t rs = rank_rsrc(rk);
 #pragma unroll
-            for (int s = 0; s < UNROLL; ++s) load_vec<IN_DT, NT>(rs, ioff[s], v[rk][s]);
+            for (int s = 0; s < UNROLL; ++s) load_vec<IN_DT, LAUX>(rs, ioff[s], v[rk][s]);
           }
 #pragma unroll
           for (int rk = 0; rk < WS; ++rk)
@@ -167,7 +174,7 @@ __global__ __launch_bounds__(256) void reduce_tiles_vec_kernel(const ReduceKArgs
             const __amdgpu_buffer_rsrc_t rs = rank_rsrc(rk);
             float v[UNROLL][VE];
 #pragma unroll
-            for (int s = 0; s < UNROLL; ++s) load_vec<IN_DT, NT>(rs, ioff[s], v[s]);
+            for (int s = 0; s < UNROLL; ++s) load_vec<IN_DT, LAUX>(rs, ioff[s], v[s]);
 #pragma unroll
             for (int s = 0; s < UNROLL; ++s)
 #pragma unroll
@@ -175,7 +182,7 @@ __global__ __launch_bounds__(256) void reduce_tiles_vec_kernel(const ReduceKArgs
           }
         }
 #pragma unroll
-        for (int s = 0; s < UNROLL; ++s) store_vec<OUT_DT, VE, NT>(out_rs, ooff[s], acc[s]);
+        for (int s = 0; s < UNROLL; ++s) store_vec<OUT_DT, VE, AUX_NT>(out_rs, ooff[s], acc[s]);
       }
     }
   }
