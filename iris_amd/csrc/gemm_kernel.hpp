@@ -108,6 +108,10 @@ struct GemmCfg {
   static constexpr int L = A_LOADS + B_LOADS;
   static constexpr int KSUB = BK / 16;
   static constexpr bool AGPR_ACC = IM * IN * 16 > 128;  // accumulators pinned to AGPRs
+  // Waves per SIMD the register budget is sized for.  A 4-wave group whose
+  // accumulators fit the 256-register half runs two groups per CU, so that one
+  // group's epilogue and barriers overlap the other's MFMA work.
+  static constexpr int WPE = AGPR_ACC ? 1 : 2;
   // wave-private epilogue scratch: 32 rows x TN 16-bit elements
   static constexpr int WS_PITCH = TN * 2;
   static constexpr int WS_BYTES = 32 * WS_PITCH;
@@ -218,7 +222,7 @@ struct Loader {
     const int blk = (isA ? I : I - Cfg::A_LOADS) * Cfg::NW + wave;
     IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + blk * 1024;
     const uint32_t off = (k0 + kcol[I] < k_limit) ? voff[I] : 0x80000000u;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, k0 * 2, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, (p.debug & 8) ? 0 : k0 * 2, 0, 0);
   }
   template <int I = 0>
   __device__ inline void issue(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
@@ -389,8 +393,18 @@ __device__ inline void atomic_add16_pair(IRIS_GLOBAL unsigned int* p, unsigned i
 //
 // OP_STORE16 : 16-bit elements of type ODT        OP_STORE32 : fp32 elements
 // OP_ATOMIC32: fp32 atomic add                    OP_ATOMIC16: 16-bit atomic add
+//
+// Returns true when the wave issued exactly FAST_STORES memory instructions
+// (every block took the 16-byte path to a single destination rank).
+template <class Cfg, int OP>
+struct StoreCount {
+  static constexpr bool F32 = (OP == OP_STORE32 || OP == OP_ATOMIC32);
+  static constexpr int NPASS = F32 ? 2 : 1;
+  static constexpr int NV = 32 / (64 / Cfg::U16);
+  static constexpr int FAST_STORES = Cfg::IM * NPASS * NV;
+};
 template <class Cfg, int OP, int ODT>
-__device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM][Cfg::IN], IRIS_LDS char* ws,
+__device__ inline bool store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM][Cfg::IN], IRIS_LDS char* ws,
                                  int wm0, int wn0, int m_end, int n_end, int lane) {  // lane: by value, see below
   constexpr bool F32 = (OP == OP_STORE32 || OP == OP_ATOMIC32);
   constexpr int ES = F32 ? 4 : 2;
@@ -405,6 +419,7 @@ __device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM
   const int lrow = lane & 31, lhalf = lane >> 5;
   const int r_begin = p.dest_all ? 0 : p.cur_rank;
   const int r_end = p.dest_all ? p.ws : p.cur_rank + 1;
+  bool all_fast = (OP == OP_STORE16 || OP == OP_STORE32) && p.vec_out && r_end - r_begin == 1;
 #pragma unroll
   for (int i = 0; i < Cfg::IM; ++i) {
 #pragma unroll
@@ -430,6 +445,7 @@ __device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM
       // ---- scratch -> memory
       const int row0 = wm0 + i * 32, col0 = wn0 + ps * CP;
       const bool interior = (row0 + 32 <= m_end) && (col0 + CP <= n_end);
+      all_fast = all_fast && interior;
 #pragma nounroll
       for (int r = r_begin; r < r_end; ++r) {
         IRIS_GLOBAL char* dst = rank_ptr(p, p.out, r);
@@ -479,7 +495,10 @@ __device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM
               off[t] = (int)((row * p.som + u * EPV) * ES);
             }
             // write-through at the flags' scope: sc1 (agent) or sc0 sc1 (system)
-            if (p.sys) {
+            if (p.debug & 32) {
+#pragma unroll
+              for (int t = 0; t < NV; ++t) __builtin_amdgcn_raw_buffer_store_b128(v[t], rs, off[t], 0, 0);
+            } else if (p.sys) {
 #pragma unroll
               for (int t = 0; t < NV; ++t) __builtin_amdgcn_raw_buffer_store_b128(v[t], rs, off[t], 0, 17);
             } else {
@@ -512,6 +531,7 @@ __device__ inline void store_acc(const GemmKArgs& p, const f32x16 (&acc)[Cfg::IM
       }
     }
   }
+  return all_fast;
 }
 
 // Publish a finished logical tile: +1 on the tile's flag of every rank
@@ -579,7 +599,8 @@ __device__ inline void mma_rest(f32x16 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg
 // ---------------------------------------------------------------------------
 
 template <class Cfg, int OP, int ODT>
-__global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArgs p) {
+__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::WPE, Cfg::WPE))) void
+gemm_persistent_kernel(const GemmKArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   IRIS_LDS char* lds = (IRIS_LDS char*)lds_raw;
 
@@ -618,6 +639,12 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArg
   // K-step, where the whole group waits on its memory counter anyway.
   const bool defer_publish = Cfg::DMA && nk > 0 && p.flag_mode != 0;
   int pending_tile = -1;
+  // 1: the pending tile's stores are exactly the FAST_STORES youngest memory
+  // operations of this wave, so the next hand-over can wait for the loads
+  // issued before them and leave the stores in flight one K-step longer
+  int pending_skip = 0;
+  constexpr int FAST_STORES = StoreCount<Cfg, OP>::FAST_STORES;
+  static_assert(Cfg::L * (Cfg::S > 2 ? Cfg::S - 2 : 0) + FAST_STORES <= 63, "vmcnt immediate");
 
   int c_item = 0;  // compute cursor
   Item c_it;
@@ -630,12 +657,22 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArg
       // let the last one (16 passes at most) retire before its result is read
       asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15");
     }
+    if (defer_publish && pending_tile >= 0) {
+      // a one-step tile: the previous tile has not been published yet
+      IRIS_WAIT_VMCNT(0);
+      __syncthreads();
+      if (tid == 0) publish_tile(p, pending_tile);
+      pending_tile = -1;
+    }
+    bool fast = false;
     if (!(p.debug & 4))
-      store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end, c_it.n_end,
-                              lane);
+      fast = store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end,
+                                     c_it.n_end, lane);
     if (c_it.last_sub) {
       if (defer_publish) {
         pending_tile = __builtin_amdgcn_readfirstlane(c_it.tile_id);
+        // the count only holds for a tile that is a single compute tile
+        pending_skip = (fast && c_it.first_sub && !(p.debug & 64)) ? 1 : 0;
       } else if (p.flag_mode != 0) {
         IRIS_WAIT_VMCNT(0);  // this wave's stores of the tile have completed
         __syncthreads();
@@ -732,15 +769,22 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_persistent_kernel(const GemmKArg
         // hand-over of stage g+1: wait for this wave's part of its slab
         // (S-2 younger slabs may stay in flight), then meet the other waves
         const int pend = __builtin_amdgcn_readfirstlane(pending_tile);
-        if (pend >= 0) {
+        const int skip = __builtin_amdgcn_readfirstlane(pending_skip);
+        if (pend >= 0 && skip == 0) {
           IRIS_WAIT_VMCNT(0);  // the previous tile's stores, too
+        } else if (pend >= 0) {
+          IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2) + FAST_STORES);  // the stores stay in flight
         } else {
           IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
         }
         block_barrier_raw();
         if (pend >= 0) {
-          if (tid == 0) publish_tile(p, pend);
-          pending_tile = -1;
+          if (skip == 0) {
+            if (tid == 0) publish_tile(p, pend);
+            pending_tile = -1;
+          } else {
+            pending_skip = 0;
+          }
         }
         const IRIS_LDS char* nstage = lds + ((g + 1) & (Cfg::S - 1)) * Cfg::STAGE;
         // fragment fetches of (g+1, substep 0), two per MFMA

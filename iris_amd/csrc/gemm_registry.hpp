@@ -48,7 +48,9 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   X(DT, OP, 256, 256, 32, 2, 4, 4, true, "256x256x32_w2x4_s4")   \
   X(DT, OP, 256, 128, 32, 2, 4, 4, true, "256x128x32_w2x4_s4")   \
   X(DT, OP, 256, 128, 64, 2, 4, 2, true, "256x128x64_w2x4_s2")   \
-  X(DT, OP, 256, 128, 64, 2, 2, 2, true, "256x128x64_w2x2_s2")
+  X(DT, OP, 256, 128, 64, 2, 2, 2, true, "256x128x64_w2x2_s2")   \
+  X(DT, OP, 256, 128, 32, 2, 2, 2, true, "256x128x32_w2x2_s2")   \
+  X(DT, OP, 128, 256, 32, 2, 2, 2, true, "128x256x32_w2x2_s2")
 
 #define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, NAME) \
   make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP>(NAME),
