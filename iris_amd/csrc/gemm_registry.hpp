@@ -34,23 +34,20 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 // wins.  `variant` k > 0 in iris_gemm_args forces entry k-1 (tuning runs).
 #define IRIS_GEMM_VARIANTS(X, DT, OP)                            \
   X(DT, OP, 256, 256, 64, 2, 4, 2, true, "256x256x64_w2x4_s2")   \
-  X(DT, OP, 256, 128, 32, 2, 2, 4, true, "256x128x32_w2x2_s4")   \
-  X(DT, OP, 128, 256, 32, 2, 2, 4, true, "128x256x32_w2x2_s4")   \
-  X(DT, OP, 128, 128, 32, 2, 2, 4, true, "128x128x32_w2x2_s4")   \
-  X(DT, OP, 256, 64, 32, 4, 1, 4, true, "256x64x32_w4x1_s4")     \
-  X(DT, OP, 64, 64, 32, 2, 2, 4, true, "64x64x32_w2x2_s4")       \
+  X(DT, OP, 256, 128, 64, 2, 2, 2, true, "256x128x64_w2x2_s2")   \
+  X(DT, OP, 128, 256, 64, 1, 4, 2, true, "128x256x64_w1x4_s2")   \
+  X(DT, OP, 128, 128, 64, 2, 2, 4, true, "128x128x64_w2x2_s4")   \
+  X(DT, OP, 256, 64, 64, 4, 1, 2, true, "256x64x64_w4x1_s2")     \
+  X(DT, OP, 64, 64, 64, 2, 2, 4, true, "64x64x64_w2x2_s4")       \
   X(DT, OP, 64, 64, 32, 2, 2, 1, false, "64x64x32_w2x2_generic")
 
-// extra variants of the headline tile, compiled for the bf16 store op only
+// extra variants, compiled for the bf16 store op only (tuning runs, and the
+// one-substep stage whose fragment buffers alternate from step to step)
 #define IRIS_GEMM_TUNING_VARIANTS(X, DT, OP)                     \
-  X(DT, OP, 256, 256, 32, 2, 2, 4, true, "256x256x32_w2x2_s4")   \
-  X(DT, OP, 256, 256, 64, 2, 2, 2, true, "256x256x64_w2x2_s2")   \
-  X(DT, OP, 256, 256, 32, 2, 4, 4, true, "256x256x32_w2x4_s4")   \
   X(DT, OP, 256, 128, 32, 2, 4, 4, true, "256x128x32_w2x4_s4")   \
   X(DT, OP, 256, 128, 64, 2, 4, 2, true, "256x128x64_w2x4_s2")   \
-  X(DT, OP, 256, 128, 64, 2, 2, 2, true, "256x128x64_w2x2_s2")   \
-  X(DT, OP, 256, 128, 32, 2, 2, 2, true, "256x128x32_w2x2_s2")   \
-  X(DT, OP, 128, 256, 32, 2, 2, 2, true, "128x256x32_w2x2_s2")
+  X(DT, OP, 128, 256, 64, 2, 4, 2, true, "128x256x64_w2x4_s2")   \
+  X(DT, OP, 128, 128, 32, 2, 2, 4, true, "128x128x32_w2x2_s4")
 
 #define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, NAME) \
   make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP>(NAME),
