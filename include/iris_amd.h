@@ -200,6 +200,18 @@ int iris_tile_schedule_launch(int32_t* out, int32_t M, int32_t N, int32_t block_
 void iris_tile_map_host(int32_t tile_id, int32_t M, int32_t N, int32_t block_m, int32_t block_n,
                         int32_t group_size_m, int32_t* pid_m, int32_t* pid_n);
 
+/*
+ * Measurement aid; no counterpart in the reference.  `num_groups` workgroups of
+ * 8 waves each run `iters` rounds of 16 v_mfma_f32_16x16x32 (ab_dtype: F16 or
+ * BF16) per wave on operands read once from `operands` (64 KiB, 16-byte
+ * aligned, any bit patterns), with nothing but registers inside the loop:
+ * num_groups * 8 * iters * 16 * 16384 FLOP per launch.  `sink` receives one
+ * float per thread (num_groups * 512).  Timed by the caller, it gives the rate
+ * the matrix cores sustain on such data under the board's power limit.
+ */
+int iris_mfma_probe_launch(const void* operands, float* sink, int32_t ab_dtype, int32_t iters, int32_t num_groups,
+                           void* stream);
+
 /* Library version, bumped when a signature in this header changes. */
 int iris_amd_abi_version(void);
 

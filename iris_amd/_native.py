@@ -131,6 +131,7 @@ SIGNATURES = {
     "iris_memset_i32_launch": (_I, [_P, ctypes.c_int32, ctypes.c_int64, _P]),
     "iris_tile_schedule_launch": (_I, [_P] + [ctypes.c_int32] * 7 + [_P]),
     "iris_tile_map_host": (None, [ctypes.c_int32] * 6 + [ctypes.POINTER(ctypes.c_int32)] * 2),
+    "iris_mfma_probe_launch": (_I, [_P, _P, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P]),
     "iris_amd_abi_version": (_I, []),
 }
 ALLOCATOR_SYMBOLS = ("finegrained_hipMalloc", "finegrained_hipFree")

@@ -421,7 +421,12 @@ __device__ inline bool store_acc(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM]
       // ---- scratch -> memory
       const int row0 = wm0 + i * 32, col0 = wn0 + ps * CP;
       const bool interior = (row0 + 32 <= m_end) && (col0 + CP <= n_end);
-      all_fast = all_fast && interior;
+      // The 16-byte store path also takes ragged blocks whose valid columns
+      // are whole 16-byte units: rows past m_end fall outside the block's
+      // buffer descriptor and units past n_end are parked out of range.
+      const int rows_ok = min(32, m_end - row0), cols_ok = min(CP, n_end - col0);
+      const bool vec_block = (OP == OP_STORE16 || OP == OP_STORE32) && (cols_ok <= 0 || cols_ok % EPV == 0);
+      all_fast = all_fast && (interior || vec_block);
 #pragma nounroll
       for (int r = r_begin; r < r_end; ++r) {
         IRIS_GLOBAL char* dst = rank_ptr(p, p.out, r);
@@ -440,7 +445,7 @@ __device__ inline bool store_acc(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM]
               __hip_atomic_fetch_add((IRIS_GLOBAL float*)(dst + ((int64_t)m * p.som + (int64_t)n * p.son) * 4),
                                      v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
-        } else if (interior && p.vec_out) {
+        } else if ((interior || vec_block) && p.vec_out) {
           if constexpr (OP == OP_ATOMIC16) {
             // one packed pair per lane, lanes along the row
             constexpr int ITER = 32 * (CP / 2) / 64;
@@ -458,8 +463,10 @@ __device__ inline bool store_acc(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM]
             constexpr int RPI = 64 / Cfg::U16;  // rows per wave-wide 16-byte read
             constexpr int NV = 32 / RPI;
             // the 32 x CP block as a buffer: rows are p.som elements apart
+            const bool any = rows_ok > 0 && cols_ok > 0;
             const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-                (void*)(dst + ((int64_t)row0 * p.som + col0) * ES), 0, (int)((31 * p.som + CP) * ES), 0x00020000);
+                (void*)(dst + ((int64_t)row0 * p.som + col0) * ES), 0,
+                any ? (int)(((rows_ok - 1) * p.som + cols_ok) * ES) : 0, 0x00020000);
             u32x4 v[NV];
             int off[NV];
 #pragma unroll
@@ -468,7 +475,7 @@ __device__ inline bool store_acc(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM]
               const int u = lane % Cfg::U16;
               const int pu = u ^ ((row / Cfg::ERPB) % Cfg::U16);
               v[t] = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + row * Cfg::WS_PITCH + pu * 16);
-              off[t] = (int)((row * p.som + u * EPV) * ES);
+              off[t] = (u + 1) * EPV <= cols_ok ? (int)((row * p.som + u * EPV) * ES) : (int)0x80000000;
             }
             // write-through at the flags' scope: sc1 (agent) or sc0 sc1 (system)
             if (p.debug & 32) {

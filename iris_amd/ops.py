@@ -293,6 +293,22 @@ def tile_map_host(tile_id, M, N, BLK_M, BLK_N, gsize_m):
     return pm.value, pn.value
 
 
+def mfma_probe(operands, sink, iters, num_groups):
+    """Launch the register-only MFMA loop (a measurement aid): returns the FLOP
+    count of the launch.  ``operands``: >= 64 KiB of fp16/bf16 on the device,
+    ``sink``: >= num_groups * 512 floats."""
+    if operands.dtype not in _DTYPES or operands.dtype == torch.float32:
+        raise ValueError("operands must be fp16 or bf16")
+    if operands.numel() * operands.element_size() < 65536 or sink.numel() < num_groups * 512:
+        raise ValueError("operands: at least 64 KiB; sink: at least num_groups * 512 floats")
+    if sink.dtype != torch.float32 or not operands.is_contiguous():
+        raise ValueError("sink must be fp32 and operands contiguous")
+    stream = torch.cuda.current_stream(operands.device).cuda_stream
+    _native.hip_try(_native.lib().iris_mfma_probe_launch(_ptr(operands), _ptr(sink), _DTYPES[operands.dtype], iters,
+                                                         num_groups, ctypes.c_void_p(stream)))
+    return num_groups * 8 * iters * 16 * 16384
+
+
 def signal_tiles(tile_completed, heap_bases, total_tiles, rank, world_size, *, include_self=False,
                  scope=SCOPE_AGENT):
     """+1 (release) on the flag of every tile on the other ranks (on every rank
