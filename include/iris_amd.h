@@ -74,6 +74,11 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 #define IRIS_DTYPE_F32 0
 #define IRIS_DTYPE_F16 1
 #define IRIS_DTYPE_BF16 2
+/* integer element types: only iris_rma_selftest_launch takes them */
+#define IRIS_DTYPE_I8 3
+#define IRIS_DTYPE_I16 4
+#define IRIS_DTYPE_I32 5
+#define IRIS_DTYPE_I64 6
 
 /* epilogues of the persistent shard GEMM */
 #define IRIS_EPI_ALL_SCATTER 0 /* examples/07_gemm_all_scatter/gemm_all_scatter.py:209-251 */
@@ -88,6 +93,7 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 /* flag scopes */
 #define IRIS_SCOPE_AGENT 0  /* all "ranks" live on this GPU */
 #define IRIS_SCOPE_SYSTEM 1 /* the reference's scope="sys" */
+#define IRIS_SCOPE_WORKGROUP 2 /* scope="cta"; only iris_rma_selftest_launch takes it */
 
 /* status word values (max-reduced by the kernels into *status) */
 #define IRIS_STATUS_OK 0
@@ -211,6 +217,38 @@ void iris_tile_map_host(int32_t tile_id, int32_t M, int32_t N, int32_t block_m, 
  */
 int iris_mfma_probe_launch(const void* operands, float* sink, int32_t ab_dtype, int32_t iters, int32_t num_groups,
                            void* stream);
+
+/*
+ * Device-side remote access (include/iris_device.hpp, the HIP counterpart of
+ * iris/iris.py:317-521) exercised the way the reference's unit tests exercise
+ * the Triton functions: one workgroup, lane i < block_size owns element i of
+ * `data` / `results` (buffers at the same heap offset on every rank), and every
+ * rank 0..num_ranks-1 is the target in turn.
+ *   LOAD        results[i]  = sum over ranks of load(data + i)      tests/unittests/test_load.py:8-31
+ *   STORE       store(results + i, data[i]) on every rank           tests/unittests/test_store.py:8-30
+ *   GET         get(data + i -> results + i), accumulate, store     tests/unittests/test_get.py:8-31
+ *   PUT         put(data + i -> results + i) on every rank          tests/unittests/test_put.py:8-26
+ *   ATOMIC_ADD  atomic_add(results + i, 1) on every rank            tests/unittests/test_atomic_add.py:8-30
+ *   ATOMIC_SUB  atomic_sub(results + i, 1) on every rank            (iris/iris.py:452-473; no reference test)
+ *   ATOMIC_CAS  atomic_cas(results, 0 -> num_ranks) on every rank   tests/unittests/test_atomic_cas.py:8-24
+ *   ATOMIC_XCHG atomic_xchg(results, num_ranks) on every rank       tests/unittests/test_atomic_xchg.py:8-23
+ * sem / scope only matter for the atomics.  block_size is 1..64; int8 has no atomics.
+ */
+#define IRIS_RMA_LOAD 0
+#define IRIS_RMA_STORE 1
+#define IRIS_RMA_GET 2
+#define IRIS_RMA_PUT 3
+#define IRIS_RMA_ATOMIC_ADD 4
+#define IRIS_RMA_ATOMIC_SUB 5
+#define IRIS_RMA_ATOMIC_CAS 6
+#define IRIS_RMA_ATOMIC_XCHG 7
+#define IRIS_SEM_RELAXED 0
+#define IRIS_SEM_ACQUIRE 1
+#define IRIS_SEM_RELEASE 2
+#define IRIS_SEM_ACQ_REL 3
+int iris_rma_selftest_launch(int32_t op, int32_t dtype, int32_t sem, int32_t scope, const void* data, void* results,
+                             const uint64_t* heap_bases, int32_t cur_rank, int32_t num_ranks, int32_t block_size,
+                             void* stream);
 
 /* Library version, bumped when a signature in this header changes. */
 int iris_amd_abi_version(void);

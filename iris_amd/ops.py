@@ -49,6 +49,14 @@ __all__ = [
 
 _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
 
+# iris_rma_selftest_launch (include/iris_amd.h)
+RMA_OPS = {"load": 0, "store": 1, "get": 2, "put": 3, "atomic_add": 4, "atomic_sub": 5, "atomic_cas": 6,
+           "atomic_xchg": 7}
+RMA_SEMS = {"relaxed": 0, "acquire": 1, "release": 2, "acq_rel": 3}
+RMA_SCOPES = {"cta": 2, "gpu": SCOPE_AGENT, "sys": SCOPE_SYSTEM}
+_RMA_DTYPES = dict(_DTYPES)
+_RMA_DTYPES.update({torch.int8: 3, torch.int16: 4, torch.int32: 5, torch.int64: 6})
+
 
 def cdiv(a: int, b: int) -> int:
     return (a + b - 1) // b
@@ -307,6 +315,24 @@ def mfma_probe(operands, sink, iters, num_groups):
     _native.hip_try(_native.lib().iris_mfma_probe_launch(_ptr(operands), _ptr(sink), _DTYPES[operands.dtype], iters,
                                                          num_groups, ctypes.c_void_p(stream)))
     return num_groups * 8 * iters * 16 * 16384
+
+
+def rma_selftest(op, data, results, heap_bases, rank, num_ranks, block_size, *, sem="acq_rel", scope="sys"):
+    """Run one of the unit-test kernels over the device-side remote-access
+    functions (include/iris_device.hpp) as rank ``rank``: ``op`` is a key of
+    ``RMA_OPS``, ``sem`` / ``scope`` the reference's strings
+    (tests/unittests/test_atomic_add.py:44-60)."""
+    if results.dtype not in _RMA_DTYPES:
+        raise ValueError(f"unsupported element type {results.dtype}")
+    if data is not None and data.dtype != results.dtype:
+        raise ValueError("data and results must have the same element type")
+    if not 1 <= block_size <= 64 or results.numel() < block_size or (data is not None and data.numel() < block_size):
+        raise ValueError("block_size must be 1..64 and fit the buffers")
+    _check_heap_bases(heap_bases, num_ranks, results.device)
+    stream = torch.cuda.current_stream(results.device).cuda_stream
+    _native.hip_try(_native.lib().iris_rma_selftest_launch(
+        RMA_OPS[op], _RMA_DTYPES[results.dtype], RMA_SEMS[sem], RMA_SCOPES[scope], _ptr(data), _ptr(results),
+        _ptr(heap_bases), rank, num_ranks, block_size, ctypes.c_void_p(stream)))
 
 
 def signal_tiles(tile_completed, heap_bases, total_tiles, rank, world_size, *, include_self=False,
