@@ -299,16 +299,19 @@ def run_decoder(args):
             hoff = shmem.heap_offset
             flags_up = shmem.zeros((t_up,), dtype=torch.int32)
             flags_dn = shmem.zeros((t_dn,), dtype=torch.int32)
-            grid_up, grid_dn = min(256, t_up), min(256, t_dn)
+            grid_up = grid_dn = 256
+            # the wrappers' P / locks buffers: with them the launcher may split K over idle programs
+            P = shmem.zeros((256, bm * bn), dtype=torch.float32)
+            locks = shmem.zeros((256,), dtype=torch.int32)
 
             def up():
                 ops.gemm_launch(x, wg.T, None, shmem.on_rank(gate_all, rank), shmem.on_rank(flags_up, rank), hb, rank,
-                                ws, grid_up, bm, bn, 64, 4, ops.EPI_ALL_SCATTER, notify=True)
+                                ws, grid_up, bm, bn, 64, 4, ops.EPI_ALL_SCATTER, notify=True, partials=P, locks=locks)
 
             def down():
                 ops.gemm_launch(h, wd.T, shmem.on_rank(part, rank), shmem.on_rank(out, rank),
                                 shmem.on_rank(flags_dn, rank), hb, rank, ws, grid_dn, bm, bn, 64, 6,
-                                ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE)
+                                ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks)
 
             def reduce():
                 ops.one_shot_reduce(shmem.on_rank(part, rank), shmem.on_rank(out, rank),
@@ -322,16 +325,24 @@ def run_decoder(args):
             got = shmem.on_rank(gate_all, 5)[:, rank * ffn:(rank + 1) * ffn].float()
             assert torch.allclose(got, ref_up, rtol=1e-2, atol=1e-2), "gate/up scatter differs from the fp32 product"
             assert torch.allclose(shmem.on_rank(part, rank), ref_dn, rtol=1e-2, atol=1e-2), "down partial differs"
+            sk = {"gate_up": ops.gemm_split_k(x, wg.T, None, shmem.on_rank(gate_all, rank),
+                                              shmem.on_rank(flags_up, rank), hb, rank, ws, grid_up, bm, bn, 64, 4,
+                                              ops.EPI_ALL_SCATTER, partials=P, locks=locks),
+                  "down": ops.gemm_split_k(h, wd.T, shmem.on_rank(part, rank), shmem.on_rank(out, rank),
+                                           shmem.on_rank(flags_dn, rank), hb, rank, ws, grid_dn, bm, bn, 64, 6,
+                                           ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks),
+                  "reduce": 1}
             for name, fn in (("gate_up", up), ("down", down), ("reduce", reduce)):
                 ms = graph_ms(fn, 10, 10)
                 if name not in best or ms < best[name][0]:
-                    best[name] = (ms, [bm, bn])
+                    best[name] = (ms, [bm, bn], sk[name])
             shmem.heap_offset = hoff
         ms_up, ms_dn, ms_red = best["gate_up"][0], best["down"][0], best["reduce"][0]
         fl = 2.0 * Mt * hidden * ffn
         wbytes = hidden * ffn * 2
         rows.append({
             "M": Mt, "tile_up": best["gate_up"][1], "tile_down": best["down"][1], "tile_reduce": best["reduce"][1],
+            "split_k_up": best["gate_up"][2], "split_k_down": best["down"][2],
             "gate_up_us": round(ms_up * 1e3, 2), "gate_up_tflops": round(fl / ms_up / 1e9, 2),
             "gate_up_weight_GBps": round(wbytes / ms_up / 1e6, 1),
             "down_us": round(ms_dn * 1e3, 2), "down_tflops": round(fl / ms_dn / 1e9, 2),

@@ -133,6 +133,18 @@ typedef struct iris_gemm_args {
   int32_t scope;        /* IRIS_SCOPE_*                                           */
   int32_t variant;      /* 0 = default kernel choice; >0 selects a tuning variant */
   uint64_t spin_timeout_ticks; /* bound on a flag wait in 100 MHz ticks; 0 = default (2 s) */
+  /* Split-K workspace: the `P` and `locks` buffers that matmul.apply receives
+   * (matmul_wrapper.py:29-31,73-92; allocated at benchmark.py:136-142).  With both
+   * given, a launch whose tiles would leave most programs idle shares each
+   * tile's K range over several programs: partial tiles go through `partials`
+   * in fp32, `locks` (all zero before the first launch, left all zero) orders
+   * the hand-over.  Results differ from the unsplit ones only in fp32
+   * summation order. */
+  float* partials;      /* [num_sms][partials_slot_elems] fp32, or NULL           */
+  int32_t* locks;       /* int32[num_sms], or NULL                                */
+  int64_t partials_slot_elems; /* >= block_m * block_n                            */
+  int32_t split_k;      /* 0 = let the launcher decide, 1 = never, n > 1 = force n */
+  int32_t reserved0;
 } iris_gemm_args;
 
 /*
@@ -147,6 +159,8 @@ int iris_gemm_launch(const iris_gemm_args* args, void* stream);
  * (what the reference reads from kk.n_regs / kk.n_spills,
  * matmul_wrapper.py:152-155).  *spills is the scratch bytes per lane. */
 int iris_gemm_kernel_info(const iris_gemm_args* args, int* n_regs, int* n_spills);
+/* The split-K factor `iris_gemm_launch` would use for `args` (1 = unsplit). */
+int iris_gemm_split_k(const iris_gemm_args* args, int* split_k);
 
 /* Name of tuning variant `variant` (1-based) of the kernel list used for
  * (ab_dtype, fp32 output?, atomic?); hipErrorInvalidValue past the end. */

@@ -70,6 +70,11 @@ class GemmArgs(ctypes.Structure):
         ("scope", ctypes.c_int32),
         ("variant", ctypes.c_int32),
         ("spin_timeout_ticks", ctypes.c_uint64),
+        ("partials", ctypes.c_void_p),
+        ("locks", ctypes.c_void_p),
+        ("partials_slot_elems", ctypes.c_int64),
+        ("split_k", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
     ]
 
 
@@ -124,6 +129,7 @@ SIGNATURES = {
     "iris_hip_arch_name": (_I, [_I, ctypes.c_char_p, ctypes.c_size_t]),
     "iris_gemm_launch": (_I, [ctypes.POINTER(GemmArgs), _P]),
     "iris_gemm_kernel_info": (_I, [ctypes.POINTER(GemmArgs), ctypes.POINTER(_I), ctypes.POINTER(_I)]),
+    "iris_gemm_split_k": (_I, [ctypes.POINTER(GemmArgs), ctypes.POINTER(_I)]),
     "iris_gemm_variant_name": (_I, [_I, _I, _I, _I, ctypes.c_char_p, ctypes.c_size_t]),
     "iris_one_shot_reduce_launch": (_I, [ctypes.POINTER(ReduceArgs), _P]),
     "iris_signal_tiles_launch": (_I, [_P, _P, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,

@@ -59,6 +59,17 @@ struct GemmKArgs {
   int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
   int sys;           // flag atomics at system scope (else agent)
   int vec_out;       // 16-byte vector access allowed on `out`
+  // Split-K: a tile's K-steps are shared out over `split_k` programs.  Part 0
+  // owns the tile: the others leave their fp32 accumulators in `partials`
+  // (slot = global item index, `partial_stride` floats apart) and raise
+  // `locks[slot]`; the owner adds them in part order and runs the epilogue.
+  int split_k;  // >= 1
+  int split_q, split_r;  // K-steps per part: nk / split_k and nk % split_k (the first split_r parts take one more)
+  float* partials;
+  int32_t* locks;
+  int64_t partial_stride;
+  uint32_t* status;   // optional: IRIS_STATUS_SPIN_TIMEOUT when a wait for a partial gave up
+  uint64_t timeout;   // bound of that wait, 100 MHz ticks
   int debug;         // tuning experiments only (IRIS_AMD_GEMM_DEBUG): 1 = fetch nothing, 2 = every row fetches row 0, 4 = store nothing
 };
 
@@ -94,6 +105,10 @@ struct GemmCfg {
   static constexpr int A_LOADS = CM * CPR / NT, B_LOADS = CN * CPR / NT;
   static constexpr int L = A_LOADS + B_LOADS;
   static constexpr int KSUB = BK / 32;  // K-substeps (one MFMA depth) per stage
+  // Split-K is compiled into the tiles with at most 64 accumulator registers
+  // a lane: the exchange of partials needs registers the 128x64 wave tiles do
+  // not have to spare, and those tiles are picked for shapes that fill the chip.
+  static constexpr bool SPLITK = IM * IN * 4 <= 64 && KSUB % 2 == 0;
   // Waves per SIMD the register budget is sized for: 256 registers a wave.
   static constexpr int WPE = 2;
   // wave-private epilogue scratch: 32 rows x TN 16-bit elements
@@ -124,12 +139,47 @@ struct Item {
   bool first_sub;
 };
 
-template <class Cfg>
+// Split-K: item `item` of program `pid` is part `part` of tile `slot / split_k`
+// and covers K-steps [k_begin, k_end).  Kept out of Item: these live in
+// scalar registers across the K loop only where they are needed.
+struct KRange {
+  int k_begin, k_end, part, slot;
+};
+template <class Cfg, bool SPLIT>
+__device__ inline KRange k_range(const GemmKArgs& p, int pid, int item, int nk) {
+  KRange r;
+  if constexpr (SPLIT) {
+    r.slot = pid + item * p.num_sms;
+    r.part = (int)((unsigned)r.slot % (unsigned)p.split_k);
+    r.k_begin = r.part * p.split_q + min(r.part, p.split_r);
+    r.k_end = r.k_begin + p.split_q + (r.part < p.split_r ? 1 : 0);
+  } else {
+    r.slot = 0;
+    r.part = 0;
+    r.k_begin = 0;
+    r.k_end = nk;
+  }
+  return r;
+}
+
+template <class Cfg, bool SPLIT>
 __device__ inline Item decode_item(const GemmKArgs& p, int pid, int item) {
   const int subs = p.sub_m * p.sub_n;
+  Item it;
+  if constexpr (SPLIT) {
+    // one compute tile per logical tile; items are (tile, part) pairs dealt
+    // out to the programs like tiles are
+    it.tile_id = (int)((unsigned)(pid + item * p.num_sms) / (unsigned)p.split_k);
+    const TileCoord tc = tile_map(it.tile_id, p.num_pid_m, p.num_pid_n, p.G);
+    it.lm0 = it.m0 = tc.pid_m * p.BM;
+    it.ln0 = it.n0 = tc.pid_n * p.BN;
+    it.m_end = min(p.M, it.lm0 + p.BM);
+    it.n_end = min(p.N, it.ln0 + p.BN);
+    it.first_sub = it.last_sub = true;
+    return it;
+  }
   const int ti = item / subs;
   const int s = item - ti * subs;
-  Item it;
   it.tile_id = pid + ti * p.num_sms;
   const TileCoord tc = tile_map(it.tile_id, p.num_pid_m, p.num_pid_n, p.G);
   it.lm0 = tc.pid_m * p.BM;
@@ -533,11 +583,51 @@ __device__ inline void publish_tile(const GemmKArgs& p, int tile_id) {
   }
 }
 
+// Split-K hand-over of a partial tile.  The partial keeps the accumulators'
+// register order (block, thread, register): 16 bytes a lane, a wave writes or
+// reads 1 KiB at a time, and nobody else needs to understand the layout.
+template <class Cfg>
+__device__ inline void dump_partial(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM][Cfg::IN], int slot, int tid) {
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(p.partials + (int64_t)slot * p.partial_stride), 0, Cfg::CM * Cfg::CN * 4, 0x00020000);
+#pragma unroll
+  for (int i = 0; i < Cfg::IM; ++i)
+#pragma unroll
+    for (int j = 0; j < Cfg::IN; ++j)
+      // write-through to where every CU of the agent reads it
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rs,
+                                             ((i * Cfg::IN + j) * Cfg::NT + tid) * 16, 0, 16);
+}
+// acc += partials of parts [q0, q0 + GROUP) of the tile whose part 0 is `slot0`,
+// in part order; parts >= split_k read as zero.  All loads of the group are in
+// flight together.
+template <class Cfg, int GROUP>
+__device__ inline void add_partials(const GemmKArgs& p, f32x4 (&acc)[Cfg::IM][Cfg::IN], int slot0, int q0, int tid) {
+  constexpr int NB = Cfg::IM * Cfg::IN;
+  u32x4 v[GROUP][NB];
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g) {
+    const bool present = q0 + g < p.split_k;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(p.partials + (int64_t)(slot0 + (present ? q0 + g : 0)) * p.partial_stride), 0,
+        present ? Cfg::CM * Cfg::CN * 4 : 0, 0x00020000);
+#pragma unroll
+    for (int b = 0; b < NB; ++b)  // sc1: coherent at agent scope without a fence
+      v[g][b] = __builtin_amdgcn_raw_buffer_load_b128(rs, (b * Cfg::NT + tid) * 16, 0, 16);
+  }
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[b / Cfg::IN][b % Cfg::IN] += __builtin_bit_cast(f32x4, v[g][b]);
+}
+
 // ---------------------------------------------------------------------------
 // The kernel
 // ---------------------------------------------------------------------------
 
-template <class Cfg, int OP, int ODT>
+// SPLIT: the split-K build of the kernel (only launched with p.split_k > 1);
+// the plain build carries none of its code or state.
+template <class Cfg, int OP, int ODT, bool SPLIT = false>
 __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::WPE, Cfg::WPE))) void
 gemm_persistent_kernel(const GemmKArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
@@ -548,10 +638,12 @@ gemm_persistent_kernel(const GemmKArgs p) {
   const int lane = tid & 63;
   const int pid = xcd_remap(blockIdx.x, p.num_sms, p.num_xcds);
 
-  const int n_tiles = pid < p.total_tiles ? (p.total_tiles - pid + p.num_sms - 1) / p.num_sms : 0;
-  const int n_items = n_tiles * p.sub_m * p.sub_n;
+  constexpr bool split = SPLIT;
+  const int work = split ? p.total_tiles * p.split_k : p.total_tiles;  // tiles, or (tile, part) pairs
+  const int n_mine = pid < work ? (work - pid + p.num_sms - 1) / p.num_sms : 0;
+  const int n_items = split ? n_mine : n_mine * p.sub_m * p.sub_n;
   const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
-  const int total_steps = n_items * nk;
+  const int total_steps = n_items * nk;  // > 0 iff there is anything to load
 
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
   IRIS_LDS char* ws = lds + Cfg::S * Cfg::STAGE + wave * Cfg::WS_BYTES;
@@ -590,7 +682,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
 
   int c_item = 0;  // compute cursor
   Item c_it;
-  if (n_items > 0) c_it = decode_item<Cfg>(p, pid, 0);
+  if (n_items > 0) c_it = decode_item<Cfg, SPLIT>(p, pid, 0);
 
   // end of a compute tile: store it, and publish the logical tile it completes
   auto epilogue = [&]() __attribute__((always_inline)) {
@@ -600,6 +692,29 @@ gemm_persistent_kernel(const GemmKArgs p) {
       __syncthreads();
       if (tid == 0) publish_tile(p, pending_tile);
       pending_tile = -1;
+    }
+    if constexpr (SPLIT) {
+      const KRange kr = k_range<Cfg, SPLIT>(p, pid, c_item, nk);
+      if (kr.part != 0) {
+        // not the owner: leave the partial, raise the lock once every wave's
+        // stores have completed, and move on
+        dump_partial<Cfg>(p, acc, kr.slot, tid);
+        IRIS_WAIT_VMCNT(0);
+        __syncthreads();
+        if (tid == 0) flag_add_relaxed((IRIS_GLOBAL int32_t*)(p.locks + kr.slot), 1, false);
+        if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, pid, c_item);
+        return;
+      }
+      // Wait for every other part at once: lane q of the group takes part q's
+      // lock (1 -> 0, which also re-arms it for the next launch), each wait
+      // bounded; then fetch the partials a few parts at a time.
+      int ok = 1;
+      if (tid >= 1 && tid < p.split_k)
+        ok = wait_tile_flag((IRIS_GLOBAL int32_t*)(p.locks + kr.slot + tid), 2, false, p.timeout, p.status) ? 1 : 0;
+      if (__syncthreads_and(ok)) {
+        constexpr int GROUP = Cfg::IM * Cfg::IN * 4 <= 16 ? 4 : Cfg::IM * Cfg::IN * 4 <= 32 ? 2 : 1;
+        for (int q = 1; q < p.split_k; q += GROUP) add_partials<Cfg, GROUP>(p, acc, kr.slot, q, tid);
+      }
     }
     bool fast = false;
     if (!(p.debug & 4))
@@ -619,7 +734,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
         __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + c_it.tile_id),
                                (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (++c_item < n_items) c_it = decode_item<Cfg>(p, pid, c_item);
+    if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, pid, c_item);
   };
   auto stamp_begin = [&]() __attribute__((always_inline)) {
     if (p.ts_begin && c_it.first_sub && tid == 0)
@@ -639,22 +754,29 @@ gemm_persistent_kernel(const GemmKArgs p) {
     // g+2..g+S are in flight.  The load cursor runs S steps ahead of the
     // compute cursor and crosses into the next item on its own.
     Loader<Cfg> ld;
-    int l_item = 0, l_k = 0;  // load cursor
+    int l_item = 0, l_k = 0, l_kend = nk;  // load cursor
     Item l_it;
     auto advance_load_cursor = [&]() __attribute__((always_inline)) {
-      if (++l_k == nk) {
-        l_k = 0;
+      if (++l_k == l_kend) {
         if (++l_item < n_items) {
-          l_it = decode_item<Cfg>(p, pid, l_item);
+          l_it = decode_item<Cfg, SPLIT>(p, pid, l_item);
+          const KRange kr = k_range<Cfg, SPLIT>(p, pid, l_item, nk);
+          l_k = kr.k_begin;
+          l_kend = kr.k_end;
           ld.setup(p, l_it, wave, lane);
         } else {
+          l_k = 0;
+          l_kend = nk;
           ld.k_limit = 0;  // nothing left to load
         }
       }
     };
     Frags<Cfg> fr;
     if (total_steps > 0) {
-      l_it = decode_item<Cfg>(p, pid, 0);
+      l_it = decode_item<Cfg, SPLIT>(p, pid, 0);
+      const KRange kr = k_range<Cfg, SPLIT>(p, pid, 0, nk);
+      l_k = kr.k_begin;
+      l_kend = kr.k_end;
       ld.setup(p, l_it, wave, lane);
 #pragma unroll
       for (int s = 0; s < Cfg::S; ++s) {
@@ -769,7 +891,9 @@ gemm_persistent_kernel(const GemmKArgs p) {
       stamp_begin();
       run_step(g, std::true_type{});
       ++g;
-      for (int k = 1; k < nk; ++k, ++g) run_step(g, std::false_type{});
+      const KRange kr = k_range<Cfg, SPLIT>(p, pid, it, nk);
+      const int steps = kr.k_end - kr.k_begin;
+      for (int k = 1; k < steps; ++k, ++g) run_step(g, std::false_type{});
       epilogue();
     }
     IRIS_WAIT_VMCNT(0);  // no load may still be writing this group's LDS when it exits
@@ -778,7 +902,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
     Frags<Cfg> fr;
     for (int it = 0; it < n_items; ++it) {
       stamp_begin();
-      for (int k = 0; k < nk; ++k) {
+      const KRange kr = k_range<Cfg, SPLIT>(p, pid, it, nk);
+      for (int k = kr.k_begin; k < kr.k_end; ++k) {
         __syncthreads();  // previous step's readers are done with the stage
         load_slab_generic<Cfg>(p, c_it, lds, k, tid);
         __syncthreads();
@@ -787,7 +912,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
           load_all<Cfg>(lds + a_row_off + xoff[kk], lds + Cfg::A_BYTES + b_row_off + xoff[kk], fr, 0);
 #pragma unroll
           for (int i = 0; i < Cfg::IM; ++i) {
-            if (k == 0 && kk == 0)
+            if (k == kr.k_begin && kk == 0)
               mma_row<Cfg, true>(acc, fr, 0, i);
             else
               mma_row<Cfg, false>(acc, fr, 0, i);

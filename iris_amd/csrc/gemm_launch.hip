@@ -181,14 +181,55 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   k.sub_m = (span_m + pick->cm - 1) / pick->cm;
   k.sub_n = (span_n + pick->cn - 1) / pick->cn;
   plan->entry = pick;
+
+  // Split-K.  The owner of a tile waits for the programs that hold its other
+  // parts, so every (tile, part) pair needs a program of its own that is
+  // resident at the same time: one pair per program, and no more programs
+  // than the device has CUs.
+  k.split_k = 1;
+  k.split_q = k.split_r = 0;
+  k.partials = a.partials;
+  k.locks = a.locks;
+  k.partial_stride = a.partials_slot_elems;
+  k.status = a.status;
+  k.timeout = a.spin_timeout_ticks ? a.spin_timeout_ticks : 200000000ull;  // 2 s at 100 MHz
+  if (a.split_k < 0) return hipErrorInvalidValue;
+  if (a.split_k != 1 && a.partials && a.locks) {
+    const int nk = (a.K + pick->bk - 1) / pick->bk;
+    int cus = 0, dev = 0;
+    const bool resident = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 && a.num_sms <= cus;
+    const bool possible = resident && pick->splitk && pick->fn_split && k.sub_m == 1 && k.sub_n == 1 &&
+                          a.partials_slot_elems >= (int64_t)pick->cm * pick->cn &&
+                          (reinterpret_cast<uintptr_t>(a.partials) & 15) == 0 && (a.partials_slot_elems % 4) == 0;
+    if (a.split_k > 1) {
+      if (!possible || a.split_k > nk || a.split_k > 64 || (int64_t)k.total_tiles * a.split_k > a.num_sms)
+        return hipErrorInvalidValue;
+      k.split_k = a.split_k;
+    } else if (possible && k.total_tiles * 2 <= a.num_sms && nk >= 32) {
+      // The hand-over of partials costs about as much as ten K-steps of a
+      // small tile, so only long K loops are split: as many parts as there
+      // are idle programs, at least four K-steps each.
+      int sk = a.num_sms / k.total_tiles;
+      if (sk > nk / 4) sk = nk / 4;
+      if (sk > 16) sk = 16;
+      if (sk > 1) k.split_k = sk;
+    }
+  } else if (a.split_k > 1) {
+    return hipErrorInvalidValue;  // forced, but no workspace
+  }
+  if (k.split_k > 1) {
+    const int nk = (a.K + pick->bk - 1) / pick->bk;
+    k.split_q = nk / k.split_k;
+    k.split_r = nk % k.split_k;
+  }
   return hipSuccess;
 }
 
-hipError_t ensure_lds(const GemmKernelEntry* e) {
+hipError_t ensure_lds(const GemmKernelEntry* e, GemmKernelFn fn) {
   // dynamic LDS above 64 KiB must be opted into once per function
   static std::mutex m;
   std::lock_guard<std::mutex> lock(m);
-  return hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                              e->lds_bytes);
 }
 
@@ -234,14 +275,15 @@ extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (plan.entry) {
     const GemmKernelEntry* e = plan.entry;
+    const GemmKernelFn fn = plan.k.split_k > 1 ? e->fn_split : e->fn;
     if (e->lds_bytes > 64 * 1024) {
-      err = ensure_lds(e);
+      err = ensure_lds(e, fn);
       if (err != hipSuccess) return err;
     }
     if (dbg())
       std::fprintf(stderr, "[iris_amd] gemm %s M=%d N=%d K=%d tiles=%d grid=%d sub=%dx%d lds=%d\n", e->name, plan.k.M,
                    plan.k.N, plan.k.K, plan.k.total_tiles, plan.k.num_sms, plan.k.sub_m, plan.k.sub_n, e->lds_bytes);
-    hipLaunchKernelGGL(e->fn, dim3(plan.k.num_sms), dim3(e->threads), e->lds_bytes, s, plan.k);
+    hipLaunchKernelGGL(fn, dim3(plan.k.num_sms), dim3(e->threads), e->lds_bytes, s, plan.k);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
   }
@@ -253,6 +295,15 @@ extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
     const iris_reduce_args r = reduce_args_from(*args);
     return iris_one_shot_reduce_launch(&r, stream);
   }
+  return hipSuccess;
+}
+
+extern "C" int iris_gemm_split_k(const iris_gemm_args* args, int* split_k) {
+  if (!args || !split_k) return hipErrorInvalidValue;
+  Plan plan;
+  hipError_t err = make_plan(*args, &plan);
+  if (err != hipSuccess) return err;
+  *split_k = plan.entry ? plan.k.split_k : 1;
   return hipSuccess;
 }
 

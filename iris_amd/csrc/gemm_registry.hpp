@@ -15,18 +15,28 @@ struct GemmKernelEntry {
   int cm, cn;  // compute tile
   int bk, wm, wn, stages;
   bool dma;    // LDS-DMA loader (needs K-contiguous, 16-byte aligned operands)
+  bool splitk;  // the kernel can share a tile's K range with other programs
   int threads;
   int lds_bytes;
   GemmKernelFn fn;
+  GemmKernelFn fn_split;  // split-K build, or null
   const char* name;
 };
+
+template <class Cfg, int OP, int ODT>
+constexpr GemmKernelFn split_fn() {
+  if constexpr (Cfg::SPLITK)
+    return &gemm_persistent_kernel<Cfg, OP, ODT, true>;
+  else
+    return nullptr;
+}
 
 template <class Cfg, int OP>
 constexpr GemmKernelEntry make_entry(const char* name) {
   constexpr int ODT = (OP == OP_STORE32 || OP == OP_ATOMIC32) ? IRIS_DTYPE_F32 : Cfg::DT;
   return GemmKernelEntry{Cfg::DT, OP,      Cfg::CM, Cfg::CN, Cfg::BK,        Cfg::WM,
-                         Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::NT, Cfg::LDS_BYTES, &gemm_persistent_kernel<Cfg, OP, ODT>,
-                         name};
+                         Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::NT, Cfg::LDS_BYTES,
+                         &gemm_persistent_kernel<Cfg, OP, ODT, false>, split_fn<Cfg, OP, ODT>(), name};
 }
 
 // The variants, in the launcher's order of preference: the first entry whose

@@ -24,6 +24,15 @@ from . import ops
 __all__ = ["make_matmul", "matmul_all_scatter", "matmul_atomics_all_reduce", "matmul_one_shot_all_reduce"]
 
 
+def _workspace_ok(P, locks, programs, BLK_M, BLK_N):
+    """Whether the caller's P / locks buffers (benchmark.py:136-142) can serve
+    as the split-K workspace: fp32 [programs, BLK_M*BLK_N] and int32 [programs]."""
+    return (isinstance(P, torch.Tensor) and isinstance(locks, torch.Tensor) and P.is_cuda and locks.is_cuda
+            and P.dtype == torch.float32 and locks.dtype == torch.int32 and P.dim() == 2 and P.is_contiguous()
+            and locks.is_contiguous() and P.shape[0] >= programs and locks.numel() >= programs
+            and P.shape[1] >= BLK_M * BLK_N)
+
+
 def _streamk_report(M, N, K, BLK_M, BLK_N, BLK_K, programs):
     """The split the reference prints in debug mode (matmul_wrapper.py:67-102);
     its kernels never use it."""
@@ -58,6 +67,7 @@ def make_matmul(epilogue: int, name: str):
         variant = 0
         status = None            # optional int32 device word for flag-wait timeouts
         spin_timeout_ticks = 0
+        split_k = 0  # 0: the launcher decides, 1: never split K, n: exactly n parts
 
         @staticmethod
         def set_debug(debug: bool):
@@ -83,6 +93,9 @@ def make_matmul(epilogue: int, name: str):
             )
             ops.gemm_launch(
                 **launch,
+                partials=P if _workspace_ok(P, locks, total_programs_streamk, BLK_M, BLK_N) else None,
+                locks=locks if _workspace_ok(P, locks, total_programs_streamk, BLK_M, BLK_N) else None,
+                split_k=matmul.split_k,
                 scope=matmul.scope,
                 mm_begin_timestamp=mm_begin_timestamp if COLLECT_TIMESTAMPS else None,
                 mm_end_timestamp=mm_end_timestamp if COLLECT_TIMESTAMPS else None,

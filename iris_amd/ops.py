@@ -30,6 +30,7 @@ from ._native import (
 __all__ = [
     "gemm_launch",
     "gemm_kernel_info",
+    "gemm_split_k",
     "gemm_variant_name",
     "one_shot_reduce",
     "signal_tiles",
@@ -117,7 +118,7 @@ def _check_heap_bases(heap_bases, world_size, device):
 
 def _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
                     gsize_m, epilogue, phase, notify, num_xcds, scope, variant, mm_begin_timestamp,
-                    mm_end_timestamp, status, spin_timeout_ticks):
+                    mm_end_timestamp, status, spin_timeout_ticks, partials=None, locks=None, split_k=0):
     assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0], "incompatible dimensions"
     device = a.device
     M, K = a.shape
@@ -190,19 +191,42 @@ def _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_s
     args.scope = scope
     args.variant = variant
     args.spin_timeout_ticks = spin_timeout_ticks
+    # split-K workspace: the wrappers' P [num_sms, BLK_M*BLK_N] fp32 and locks [num_sms] int32
+    if (partials is None) != (locks is None):
+        raise ValueError("partials and locks go together")
+    if partials is not None:
+        _require_cuda("partials", partials, device)
+        _require_cuda("locks", locks, device)
+        if partials.dtype != torch.float32 or partials.dim() != 2 or not partials.is_contiguous():
+            raise TypeError("partials must be a contiguous fp32 matrix [num_sms, BLK_M * BLK_N]")
+        if locks.dtype != torch.int32 or not locks.is_contiguous():
+            raise TypeError("locks must be a contiguous int32 tensor")
+        if partials.shape[0] < num_sms or locks.numel() < num_sms:
+            raise ValueError("partials and locks need one slot per program")
+        args.partials, args.locks = _ptr(partials), _ptr(locks)
+        args.partials_slot_elems = partials.shape[1]
+    elif split_k > 1:
+        raise ValueError("split_k > 1 needs the partials and locks workspace")
+    args.split_k = split_k
     return args
 
 
 def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
                 gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, scope=SCOPE_AGENT, variant=0,
-                mm_begin_timestamp=None, mm_end_timestamp=None, status=None, spin_timeout_ticks=0):
+                mm_begin_timestamp=None, mm_end_timestamp=None, status=None, spin_timeout_ticks=0, partials=None,
+                locks=None, split_k=0):
     """Launch the persistent shard GEMM ``a @ b`` with a tile-publishing epilogue.
+
+    ``partials`` / ``locks`` are the wrappers' ``P`` and ``locks`` buffers
+    (matmul_wrapper.py:29-31): with them, a launch with far fewer tiles than
+    programs splits each tile's K range over several programs (``split_k`` 0:
+    the launcher decides, 1: never, n: exactly n).
 
     The kernel launch of the reference wrappers (matmul_wrapper.py:109-150).
     """
     args = _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N,
                            BLK_K, gsize_m, epilogue, phase, notify, num_xcds, scope, variant, mm_begin_timestamp,
-                           mm_end_timestamp, status, spin_timeout_ticks)
+                           mm_end_timestamp, status, spin_timeout_ticks, partials, locks, split_k)
     stream = torch.cuda.current_stream(a.device).cuda_stream
     with torch.cuda.device(a.device):
         err = _native.lib().iris_gemm_launch(ctypes.byref(args), stream)
@@ -211,6 +235,22 @@ def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size,
             "iris_gemm_launch rejected the arguments (shape, strides, dtypes, grid or rank layout it does not take)"
         )
     _native.hip_try(err)
+
+
+def gemm_split_k(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
+                 gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, variant=0, partials=None,
+                 locks=None, split_k=0):
+    """The split-K factor a launch with these arguments would use (1: unsplit)."""
+    args = _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N,
+                           BLK_K, gsize_m, epilogue, phase, notify, num_xcds, SCOPE_AGENT, variant, None, None, None,
+                           0, partials, locks, split_k)
+    sk = ctypes.c_int()
+    with torch.cuda.device(a.device):
+        err = _native.lib().iris_gemm_split_k(ctypes.byref(args), ctypes.byref(sk))
+    if err == _native.HIP_ERROR_INVALID_VALUE:
+        raise ValueError("iris_gemm_split_k rejected the arguments")
+    _native.hip_try(err)
+    return sk.value
 
 
 def gemm_kernel_info(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,

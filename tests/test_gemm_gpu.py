@@ -397,3 +397,104 @@ def test_launcher_rejects_what_the_kernels_do_not_take(shmem):
     with pytest.raises(TypeError):  # fp32 operands
         ops.gemm_launch(a.float(), b.float(), None, cg, None, None, 0, 1, 4, 64, 64, 64, 1, ops.EPI_ALL_SCATTER,
                         notify=False)
+
+
+# --------------------------------------------------------------------------- split-K
+def split_workspace(shmem, grid, BM, BN):
+    return (shmem.zeros((grid, BM * BN), dtype=torch.float32), shmem.zeros((grid,), dtype=torch.int32))
+
+
+@pytest.mark.parametrize("M,N,K,BM,BN,split_k", [
+    (100, 200, 1024, 64, 64, 2),
+    (100, 200, 1024, 64, 64, 8),
+    (16, 1376, 4096, 64, 64, 8),     # decoder gate/up at 16 tokens
+    (128, 512, 1376, 128, 128, 5),   # 22 K-steps (the last one half empty) in 5 uneven parts
+    (200, 72, 776, 256, 64, 4),
+    (1, 64, 128, 64, 64, 2),         # one K-step per part
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_split_k_all_scatter(shmem, M, N, K, BM, BN, split_k, dtype):
+    """A tile's K range shared by several programs: partials through the
+    workspace, the owner adds them, stores and publishes.  Twice in a row: the
+    locks are left re-armed."""
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    grid = 256
+    partials, locks = split_workspace(shmem, grid, BM, BN)
+    want = O.shard_gemm(A, B, dtype)
+    for launch in (1, 2):
+        cg.zero_()
+        ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, grid, BM, BN, 64, 2, ops.EPI_ALL_SCATTER, partials=partials,
+                        locks=locks, split_k=split_k)
+        torch.cuda.synchronize()
+        check_close(cg, want, f"launch {launch}")
+        assert flags.cpu().tolist() == [launch] * total
+        assert int(locks.abs().max().item()) == 0
+
+
+def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
+    dtype = torch.bfloat16
+    A, B = make_ab(16, 1376, 4096, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((16, 1376), dtype=dtype)
+    flags = shmem.zeros((32,), dtype=torch.int32)
+    partials, locks = split_workspace(shmem, 256, 64, 64)
+    common = (a, b, None, cg, flags, None, 0, 1, 256, 64, 64, 64, 4, ops.EPI_ALL_SCATTER)
+    # 22 tiles on 256 programs, 64 K-steps: 11 parts each
+    assert ops.gemm_split_k(*common, partials=partials, locks=locks) == 11
+    assert ops.gemm_split_k(*common) == 1                                    # no workspace
+    assert ops.gemm_split_k(*common, partials=partials, locks=locks, split_k=1) == 1
+    ops.gemm_launch(*common, partials=partials, locks=locks)
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, dtype))
+    assert flags.cpu().tolist()[:22] == [1] * 22 and int(locks.abs().max().item()) == 0
+    # enough tiles to fill the programs: unsplit
+    A2, B2 = make_ab(1024, 1024, 512, dtype)
+    a2, b2 = to_heap(shmem, A2), to_heap(shmem, B2)
+    cg2 = shmem.zeros((1024, 1024), dtype=dtype)
+    flags2 = shmem.zeros((256,), dtype=torch.int32)
+    assert ops.gemm_split_k(a2, b2, None, cg2, flags2, None, 0, 1, 256, 64, 64, 64, 4, ops.EPI_ALL_SCATTER,
+                            partials=partials, locks=locks) == 1
+    # a forced split the launch cannot honour is an error, not a silent fallback
+    with pytest.raises(ValueError):
+        ops.gemm_launch(*common, split_k=4)                                  # no workspace
+    with pytest.raises(ValueError):
+        ops.gemm_launch(*common, partials=partials, locks=locks, split_k=16)  # 22 * 16 pairs > 256 programs
+    with pytest.raises(ValueError):
+        ops.gemm_launch(a2, b2, None, cg2, flags2, None, 0, 1, 256, 256, 256, 64, 4, ops.EPI_ALL_SCATTER,
+                        partials=shmem.zeros((256, 256 * 256), dtype=torch.float32), locks=locks, split_k=2)
+
+
+def test_split_k_with_the_other_epilogues_and_virtual_ranks(shmem):
+    """Atomic accumulate and the one-shot producer behind a split K loop."""
+    dtype = torch.bfloat16
+    ws = 4
+    M, N, K = 64, 256, 2048
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    hb = shmem.get_heap_bases()
+    partials, locks = split_workspace(shmem, 256, 64, 64)
+    want32 = O.shard_gemm(A, B, None)
+    c32 = shmem.zeros((M, N), dtype=torch.float32)
+    for r in range(ws):
+        shmem.on_rank(c32, r).zero_()
+    ops.gemm_launch(a, b, None, shmem.on_rank(c32, 1), None, hb, 1, ws, 256, 64, 64, 64, 2, ops.EPI_ATOMIC_ADD,
+                    partials=partials, locks=locks, split_k=8)
+    torch.cuda.synchronize()
+    for r in range(ws):
+        check_close(shmem.on_rank(c32, r), want32, f"atomic add on rank {r}")
+    part = shmem.zeros((M, N), dtype=torch.float32)
+    out = shmem.zeros((M, N), dtype=dtype)
+    flags = shmem.zeros((4,), dtype=torch.int32)
+    for r in range(ws):
+        shmem.on_rank(flags, r).zero_()
+    ops.gemm_launch(a, b, shmem.on_rank(part, 2), shmem.on_rank(out, 2), shmem.on_rank(flags, 2), hb, 2, ws, 256, 64,
+                    64, 64, 2, ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=partials, locks=locks, split_k=4)
+    torch.cuda.synchronize()
+    check_close(shmem.on_rank(part, 2), want32, "one-shot partial")
+    for r in range(ws):  # the producer signals every other rank once per tile
+        assert shmem.on_rank(flags, r).cpu().tolist() == [0 if r == 2 else 1] * 4
+    assert int(locks.abs().max().item()) == 0
