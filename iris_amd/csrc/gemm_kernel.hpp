@@ -198,8 +198,11 @@ __device__ inline Item decode_item(const GemmKArgs& p, int pid, int item) {
 template <typename P>
 __device__ inline IRIS_GLOBAL P* rank_ptr(const GemmKArgs& p, P* ptr, int r) {
   if (r == p.cur_rank || p.heap_bases == nullptr) return (IRIS_GLOBAL P*)ptr;
-  // r and the bases are the same for the whole wave: keep the result scalar
-  return translate(ptr, uniform_u64(p.heap_bases[p.cur_rank]), uniform_u64(p.heap_bases[r]));
+  // r and the bases are the same for the whole wave and the table does not
+  // change while the kernel runs: scalar loads, which do not wait for stores
+  const __attribute__((address_space(4))) uint64_t* hb =
+      (const __attribute__((address_space(4))) uint64_t*)p.heap_bases;
+  return translate(ptr, uniform_u64(hb[p.cur_rank]), uniform_u64(hb[r]));
 }
 
 // ---------------------------------------------------------------------------
@@ -430,7 +433,7 @@ struct StoreCount {
   static constexpr int FAST_STORES = (Cfg::TM / 32) * NPASS * NV;
 };
 template <class Cfg, int OP, int ODT>
-__device__ inline bool store_acc(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM][Cfg::IN], IRIS_LDS char* ws,
+__device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM][Cfg::IN], IRIS_LDS char* ws,
                                  int wm0, int wn0, int m_end, int n_end, int lane) {  // lane: by value, see below
   constexpr bool F32 = (OP == OP_STORE32 || OP == OP_ATOMIC32);
   constexpr int ES = F32 ? 4 : 2;
@@ -446,124 +449,126 @@ __device__ inline bool store_acc(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM]
   const int r_begin = p.dest_all ? 0 : p.cur_rank;
   const int r_end = p.dest_all ? p.ws : p.cur_rank + 1;
   bool all_fast = (OP == OP_STORE16 || OP == OP_STORE32) && p.vec_out && r_end - r_begin == 1;
+  const bool single = r_end - r_begin == 1;
+  IRIS_GLOBAL char* dst0 = rank_ptr(p, p.out, r_begin);
+  // AUX: write-through at the flags' scope for the 16-byte stores, sc1 (agent)
+  // or sc0 sc1 (system); chosen once, outside the loops
+  auto blocks = [&](auto aux_tag) __attribute__((always_inline)) {
+    constexpr int AUX = decltype(aux_tag)::value;
 #pragma unroll
-  for (int i = 0; i < Cfg::TM / 32; ++i) {
+    for (int i = 0; i < Cfg::TM / 32; ++i) {
 #pragma unroll
-    for (int ps = 0; ps < NPASS; ++ps) {
-      // ---- registers -> scratch
+      for (int ps = 0; ps < NPASS; ++ps) {
+        // ---- registers -> scratch
 #pragma unroll
-      for (int ib = 0; ib < 2; ++ib) {
-        const int row = ib * 16 + lr;
-        const int sw = (row / Cfg::ERPB) % Cfg::U16;
+        for (int ib = 0; ib < 2; ++ib) {
+          const int row = ib * 16 + lr;
+          const int sw = (row / Cfg::ERPB) % Cfg::U16;
 #pragma unroll
-        for (int g = 0; g < NJ; ++g) {
-          const f32x4 a4 = acc[i * 2 + ib][ps * NJ + g];
-          if constexpr (F32) {
-            const int u = (g * 4 + lq) ^ sw;
-            *reinterpret_cast<IRIS_LDS f32x4*>(ws + row * Cfg::WS_PITCH + u * 16) = a4;
-          } else {
-            const int u = (g * 2 + (lq >> 1)) ^ sw;
-            const u32x2 v = {pack2<ODT>(a4[0], a4[1]), pack2<ODT>(a4[2], a4[3])};
-            *reinterpret_cast<IRIS_LDS u32x2*>(ws + row * Cfg::WS_PITCH + u * 16 + (lq & 1) * 8) = v;
+          for (int g = 0; g < NJ; ++g) {
+            const f32x4 a4 = acc[i * 2 + ib][ps * NJ + g];
+            if constexpr (F32) {
+              const int u = (g * 4 + lq) ^ sw;
+              *reinterpret_cast<IRIS_LDS f32x4*>(ws + row * Cfg::WS_PITCH + u * 16) = a4;
+            } else {
+              const int u = (g * 2 + (lq >> 1)) ^ sw;
+              const u32x2 v = {pack2<ODT>(a4[0], a4[1]), pack2<ODT>(a4[2], a4[3])};
+              *reinterpret_cast<IRIS_LDS u32x2*>(ws + row * Cfg::WS_PITCH + u * 16 + (lq & 1) * 8) = v;
+            }
           }
         }
-      }
-      // ---- scratch -> memory
-      const int row0 = wm0 + i * 32, col0 = wn0 + ps * CP;
-      const bool interior = (row0 + 32 <= m_end) && (col0 + CP <= n_end);
-      // The 16-byte store path also takes ragged blocks whose valid columns
-      // are whole 16-byte units: rows past m_end fall outside the block's
-      // buffer descriptor and units past n_end are parked out of range.
-      const int rows_ok = min(32, m_end - row0), cols_ok = min(CP, n_end - col0);
-      const bool vec_block = (OP == OP_STORE16 || OP == OP_STORE32) && (cols_ok <= 0 || cols_ok % EPV == 0);
-      all_fast = all_fast && (interior || vec_block);
+        // ---- scratch -> memory
+        const int row0 = wm0 + i * 32, col0 = wn0 + ps * CP;
+        const bool interior = (row0 + 32 <= m_end) && (col0 + CP <= n_end);
+        // The 16-byte store path also takes ragged blocks whose valid columns
+        // are whole 16-byte units: rows past m_end fall outside the block's
+        // buffer descriptor and units past n_end are parked out of range.
+        const int rows_ok = min(32, m_end - row0), cols_ok = min(CP, n_end - col0);
+        const bool vec_block = (OP == OP_STORE16 || OP == OP_STORE32) && (cols_ok <= 0 || cols_ok % EPV == 0);
+        all_fast = all_fast && (interior || vec_block);
 #pragma nounroll
-      for (int r = r_begin; r < r_end; ++r) {
-        IRIS_GLOBAL char* dst = rank_ptr(p, p.out, r);
-        if (OP == OP_ATOMIC32) {
-          // one fp32 per lane, lanes along the row
-          constexpr int ITER = 32 * CP / 64;
+        for (int r = r_begin; r < r_end; ++r) {
+          IRIS_GLOBAL char* dst = single ? dst0 : rank_ptr(p, p.out, r);
+          if (OP == OP_ATOMIC32) {
+            // one fp32 per lane, lanes along the row
+            constexpr int ITER = 32 * CP / 64;
 #pragma nounroll  // an atomic per iteration: nothing to gain, and unrolled address math spills
-          for (int t = 0; t < ITER; ++t) {
-            const int idx = t * 64 + lane;
-            const int row = idx / CP, cc = idx % CP;
-            const int u = (cc / 4) ^ ((row / Cfg::ERPB) % Cfg::U16);
-            const float v =
-                *reinterpret_cast<const IRIS_LDS float*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 4) * 4);
-            const int m = row0 + row, n = col0 + cc;
-            if (m < m_end && n < n_end)
-              __hip_atomic_fetch_add((IRIS_GLOBAL float*)(dst + ((int64_t)m * p.som + (int64_t)n * p.son) * 4),
-                                     v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-        } else if ((interior || vec_block) && p.vec_out) {
-          if constexpr (OP == OP_ATOMIC16) {
-            // one packed pair per lane, lanes along the row
-            constexpr int ITER = 32 * (CP / 2) / 64;
-#pragma nounroll
             for (int t = 0; t < ITER; ++t) {
               const int idx = t * 64 + lane;
-              const int row = idx / (CP / 2), cc = (idx % (CP / 2)) * 2;
-              const int u = (cc / 8) ^ ((row / Cfg::ERPB) % Cfg::U16);
-              const unsigned int v =
-                  *reinterpret_cast<const IRIS_LDS unsigned int*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 8) * 2);
+              const int row = idx / CP, cc = idx % CP;
+              const int u = (cc / 4) ^ ((row / Cfg::ERPB) % Cfg::U16);
+              const float v =
+                  *reinterpret_cast<const IRIS_LDS float*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 4) * 4);
               const int m = row0 + row, n = col0 + cc;
-              atomic_add16_pair<ODT>((IRIS_GLOBAL unsigned int*)(dst + ((int64_t)m * p.som + n) * 2), v);
+              if (m < m_end && n < n_end)
+                __hip_atomic_fetch_add((IRIS_GLOBAL float*)(dst + ((int64_t)m * p.som + (int64_t)n * p.son) * 4),
+                                       v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+          } else if ((interior || vec_block) && p.vec_out) {
+            if constexpr (OP == OP_ATOMIC16) {
+              // one packed pair per lane, lanes along the row
+              constexpr int ITER = 32 * (CP / 2) / 64;
+#pragma nounroll
+              for (int t = 0; t < ITER; ++t) {
+                const int idx = t * 64 + lane;
+                const int row = idx / (CP / 2), cc = (idx % (CP / 2)) * 2;
+                const int u = (cc / 8) ^ ((row / Cfg::ERPB) % Cfg::U16);
+                const unsigned int v =
+                    *reinterpret_cast<const IRIS_LDS unsigned int*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 8) * 2);
+                const int m = row0 + row, n = col0 + cc;
+                atomic_add16_pair<ODT>((IRIS_GLOBAL unsigned int*)(dst + ((int64_t)m * p.som + n) * 2), v);
+              }
+            } else {
+              constexpr int RPI = 64 / Cfg::U16;  // rows per wave-wide 16-byte read
+              constexpr int NV = 32 / RPI;
+              // the 32 x CP block as a buffer: rows are p.som elements apart
+              const bool any = rows_ok > 0 && cols_ok > 0;
+              const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+                  (void*)(dst + ((int64_t)row0 * p.som + col0) * ES), 0,
+                  any ? (int)(((rows_ok - 1) * p.som + cols_ok) * ES) : 0, 0x00020000);
+              u32x4 v[NV];
+              int off[NV];
+#pragma unroll
+              for (int t = 0; t < NV; ++t) {
+                const int row = t * RPI + lane / Cfg::U16;
+                const int u = lane % Cfg::U16;
+                const int pu = u ^ ((row / Cfg::ERPB) % Cfg::U16);
+                v[t] = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + row * Cfg::WS_PITCH + pu * 16);
+                off[t] = (u + 1) * EPV <= cols_ok ? (int)((row * p.som + u * EPV) * ES) : (int)0x80000000;
+              }
+#pragma unroll
+              for (int t = 0; t < NV; ++t) __builtin_amdgcn_raw_buffer_store_b128(v[t], rs, off[t], 0, AUX);
             }
           } else {
-            constexpr int RPI = 64 / Cfg::U16;  // rows per wave-wide 16-byte read
-            constexpr int NV = 32 / RPI;
-            // the 32 x CP block as a buffer: rows are p.som elements apart
-            const bool any = rows_ok > 0 && cols_ok > 0;
-            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-                (void*)(dst + ((int64_t)row0 * p.som + col0) * ES), 0,
-                any ? (int)(((rows_ok - 1) * p.som + cols_ok) * ES) : 0, 0x00020000);
-            u32x4 v[NV];
-            int off[NV];
-#pragma unroll
-            for (int t = 0; t < NV; ++t) {
-              const int row = t * RPI + lane / Cfg::U16;
-              const int u = lane % Cfg::U16;
-              const int pu = u ^ ((row / Cfg::ERPB) % Cfg::U16);
-              v[t] = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + row * Cfg::WS_PITCH + pu * 16);
-              off[t] = (u + 1) * EPV <= cols_ok ? (int)((row * p.som + u * EPV) * ES) : (int)0x80000000;
-            }
-            // write-through at the flags' scope: sc1 (agent) or sc0 sc1 (system)
-            if (p.debug & 32) {
-#pragma unroll
-              for (int t = 0; t < NV; ++t) __builtin_amdgcn_raw_buffer_store_b128(v[t], rs, off[t], 0, 0);
-            } else if (p.sys) {
-#pragma unroll
-              for (int t = 0; t < NV; ++t) __builtin_amdgcn_raw_buffer_store_b128(v[t], rs, off[t], 0, 17);
-            } else {
-#pragma unroll
-              for (int t = 0; t < NV; ++t) __builtin_amdgcn_raw_buffer_store_b128(v[t], rs, off[t], 0, 16);
-            }
-          }
-        } else {
-          // ragged edge or unaligned destination: element by element
+            // ragged edge or unaligned destination: element by element
 #pragma nounroll
-          for (int idx = lane; idx < 32 * CP; idx += 64) {
-            const int row = idx / CP, cc = idx % CP;
-            const int u = (cc / EPV) ^ ((row / Cfg::ERPB) % Cfg::U16);
-            const IRIS_LDS char* src = ws + row * Cfg::WS_PITCH + u * 16 + (cc % EPV) * ES;
-            const int m = row0 + row, n = col0 + cc;
-            if (m < m_end && n < n_end) {
-              IRIS_GLOBAL char* d = dst + ((int64_t)m * p.som + (int64_t)n * p.son) * ES;
-              if constexpr (OP == OP_STORE32)
-                store_through((IRIS_GLOBAL unsigned int*)d, *reinterpret_cast<const IRIS_LDS unsigned int*>(src),
-                              p.sys != 0);
-              else if constexpr (OP == OP_STORE16)
-                store_through((IRIS_GLOBAL unsigned short*)d,
-                              *reinterpret_cast<const IRIS_LDS unsigned short*>(src), p.sys != 0);
-              else
-                atomic_add16_cas<ODT>((IRIS_GLOBAL unsigned short*)d,
-                                      from16<ODT>(*reinterpret_cast<const IRIS_LDS unsigned short*>(src)));
+            for (int idx = lane; idx < 32 * CP; idx += 64) {
+              const int row = idx / CP, cc = idx % CP;
+              const int u = (cc / EPV) ^ ((row / Cfg::ERPB) % Cfg::U16);
+              const IRIS_LDS char* src = ws + row * Cfg::WS_PITCH + u * 16 + (cc % EPV) * ES;
+              const int m = row0 + row, n = col0 + cc;
+              if (m < m_end && n < n_end) {
+                IRIS_GLOBAL char* d = dst + ((int64_t)m * p.som + (int64_t)n * p.son) * ES;
+                if constexpr (OP == OP_STORE32)
+                  store_through((IRIS_GLOBAL unsigned int*)d, *reinterpret_cast<const IRIS_LDS unsigned int*>(src),
+                                p.sys != 0);
+                else if constexpr (OP == OP_STORE16)
+                  store_through((IRIS_GLOBAL unsigned short*)d,
+                                *reinterpret_cast<const IRIS_LDS unsigned short*>(src), p.sys != 0);
+                else
+                  atomic_add16_cas<ODT>((IRIS_GLOBAL unsigned short*)d,
+                                        from16<ODT>(*reinterpret_cast<const IRIS_LDS unsigned short*>(src)));
+              }
             }
           }
         }
       }
     }
-  }
+  };
+  if ((OP == OP_STORE16 || OP == OP_STORE32) && p.sys)
+    blocks(std::integral_constant<int, 17>{});
+  else
+    blocks(std::integral_constant<int, 16>{});
   return all_fast;
 }
 
