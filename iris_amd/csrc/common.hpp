@@ -51,11 +51,28 @@ __host__ __device__ inline TileCoord tile_map(int tile_id, int num_pid_m, int nu
   return t;
 }
 
+// (pid_m, pid_n) -> tile_id: the inverse of tile_map.
+__host__ __device__ inline int tile_id_of(int pid_m, int pid_n, int num_pid_m, int num_pid_n, int G) {
+  const int group_id = pid_m / G;
+  const int first_pid_m = group_id * G;
+  const int rem = num_pid_m - first_pid_m;
+  const int group_size_m = rem < G ? rem : G;
+  return group_id * G * num_pid_n + pid_n * group_size_m + (pid_m - first_pid_m);
+}
+
 // program-id remap that keeps consecutive tiles on one XCD;
 // gemm_one_shot_all_reduce.py:135-136.
 __host__ __device__ inline int xcd_remap(int pid, int num_sms, int num_xcds) {
   if (num_xcds != 1) pid = (pid % num_xcds) * (num_sms / num_xcds) + (pid / num_xcds);
   return pid;
+}
+
+// Entry r of the table of heap bases through a scalar load.  The table does
+// not change while a kernel runs, and a scalar load, unlike a vector load of
+// the same word, does not make the wave wait for its outstanding vector
+// loads and stores before the value can be used.
+__device__ inline uint64_t heap_base_at(const uint64_t* heap_bases, int r) {
+  return ((const __attribute__((address_space(4))) uint64_t*)heap_bases)[r];
 }
 
 // A 64-bit value every lane of the wave agrees on, as scalar registers.
@@ -176,6 +193,23 @@ __device__ inline bool wait_tile_flag(IRIS_GLOBAL int32_t* flag, int ws, bool sy
   for (;;) {
     const int old = flag_cas_acquire(flag, ws - 1, 0, sys);
     if (old >= ws - 1) return true;
+    if (wall_clock64() - t0 > timeout) {
+      if (status) atomicMax(status, (uint32_t)IRIS_STATUS_SPIN_TIMEOUT);
+      return false;
+    }
+    __builtin_amdgcn_s_sleep(8);
+  }
+}
+
+// Bounded wait until a tile's flag has reached `need`, without consuming it.
+// Returns whether it has; a wait that gives up records IRIS_STATUS_SPIN_TIMEOUT.
+__device__ inline bool wait_tile_ready(IRIS_GLOBAL int32_t* flag, int need, bool sys, uint64_t timeout,
+                                       uint32_t* status) {
+  const uint64_t t0 = wall_clock64();
+  for (;;) {
+    const int v = sys ? __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)
+                      : __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (v >= need) return true;
     if (wall_clock64() - t0 > timeout) {
       if (status) atomicMax(status, (uint32_t)IRIS_STATUS_SPIN_TIMEOUT);
       return false;

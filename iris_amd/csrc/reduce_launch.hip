@@ -17,8 +17,12 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 // agent, sc0 sc1 for the system), which spares the cache-invalidating fence
 // after every flag wait (~35 us over the 1024 tiles of an [8192,8192] reduce).
 template <int IN_DT, int OUT_DT>
-ReduceFn pick_vec(int ws, int variant, bool sys) {
+ReduceFn pick_vec(int ws, int variant, bool sys, bool rows) {
   constexpr int AGENT = AUX_NT | AUX_SC1, SYSTEM = AUX_NT | AUX_SC1 | AUX_SC0;
+  if (rows) {
+    if (ws == 8) return sys ? &reduce_rows_kernel<IN_DT, OUT_DT, SYSTEM, 8> : &reduce_rows_kernel<IN_DT, OUT_DT, AGENT, 8>;
+    return sys ? &reduce_rows_kernel<IN_DT, OUT_DT, SYSTEM, 0> : &reduce_rows_kernel<IN_DT, OUT_DT, AGENT, 0>;
+  }
   if (ws != 8)
     return sys ? &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 0, 2, SYSTEM> : &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 0, 2, AGENT>;
   if (sys) return &reduce_tiles_vec_kernel<IN_DT, OUT_DT, 8, 3, SYSTEM>;
@@ -34,20 +38,20 @@ ReduceFn pick_vec(int ws, int variant, bool sys) {
   }
 }
 
-ReduceFn pick(int in_dt, int out_dt, int ws, int variant, bool sys) {
+ReduceFn pick(int in_dt, int out_dt, int ws, int variant, bool sys, bool rows) {
   if (in_dt == IRIS_DTYPE_F32) {
-    if (out_dt == IRIS_DTYPE_BF16) return pick_vec<IRIS_DTYPE_F32, IRIS_DTYPE_BF16>(ws, variant, sys);
-    if (out_dt == IRIS_DTYPE_F16) return pick_vec<IRIS_DTYPE_F32, IRIS_DTYPE_F16>(ws, variant, sys);
-    return pick_vec<IRIS_DTYPE_F32, IRIS_DTYPE_F32>(ws, variant, sys);
+    if (out_dt == IRIS_DTYPE_BF16) return pick_vec<IRIS_DTYPE_F32, IRIS_DTYPE_BF16>(ws, variant, sys, rows);
+    if (out_dt == IRIS_DTYPE_F16) return pick_vec<IRIS_DTYPE_F32, IRIS_DTYPE_F16>(ws, variant, sys, rows);
+    return pick_vec<IRIS_DTYPE_F32, IRIS_DTYPE_F32>(ws, variant, sys, rows);
   }
   if (in_dt == IRIS_DTYPE_BF16) {
-    if (out_dt == IRIS_DTYPE_BF16) return pick_vec<IRIS_DTYPE_BF16, IRIS_DTYPE_BF16>(ws, variant, sys);
-    if (out_dt == IRIS_DTYPE_F32) return pick_vec<IRIS_DTYPE_BF16, IRIS_DTYPE_F32>(ws, variant, sys);
+    if (out_dt == IRIS_DTYPE_BF16) return pick_vec<IRIS_DTYPE_BF16, IRIS_DTYPE_BF16>(ws, variant, sys, rows);
+    if (out_dt == IRIS_DTYPE_F32) return pick_vec<IRIS_DTYPE_BF16, IRIS_DTYPE_F32>(ws, variant, sys, rows);
     return nullptr;
   }
   if (in_dt == IRIS_DTYPE_F16) {
-    if (out_dt == IRIS_DTYPE_F16) return pick_vec<IRIS_DTYPE_F16, IRIS_DTYPE_F16>(ws, variant, sys);
-    if (out_dt == IRIS_DTYPE_F32) return pick_vec<IRIS_DTYPE_F16, IRIS_DTYPE_F32>(ws, variant, sys);
+    if (out_dt == IRIS_DTYPE_F16) return pick_vec<IRIS_DTYPE_F16, IRIS_DTYPE_F16>(ws, variant, sys, rows);
+    if (out_dt == IRIS_DTYPE_F32) return pick_vec<IRIS_DTYPE_F16, IRIS_DTYPE_F32>(ws, variant, sys, rows);
     return nullptr;
   }
   return nullptr;
@@ -122,10 +126,44 @@ extern "C" int iris_one_shot_reduce_launch(const iris_reduce_args* a, void* stre
                    // lane offsets inside a tile are 32-bit
                    k.scm >= k.N && k.sgm >= k.N && ((int64_t)k.BM + 256) * k.scm * ies < (1ll << 31) &&
                    ((int64_t)k.BM + 256) * k.sgm * oes < (1ll << 31);
-  ReduceFn fn = vec ? pick(k.c_dt, k.cg_dt, k.ws, a->variant, k.sys != 0) : nullptr;
-  if (!fn) fn = &reduce_tiles_generic_kernel;
+  // Row bands instead of tiles (variant 7 asks for them, 8 forbids them): an
+  // item is 8192 elements per partial, whole rows when they are shorter.
+  // They pay off when a row is long, from 16 KiB of input a row ...
+  bool rows = false;
+  if (vec && a->variant != 8) {
+    const int item_vecs = ies == 4 ? 2048 : 1024;  // 16-byte strips per item: 8192 elements
+    const int nv = k.N / ve;
+    k.band_vecs = nv < item_vecs ? nv : item_vecs;
+    int br = 1;
+    if (nv < item_vecs)
+      while (br * 2 * nv <= item_vecs && k.BM % (br * 2) == 0) br *= 2;
+    k.band_rows = br;
+    k.band_chunks = (nv + k.band_vecs - 1) / k.band_vecs;
+    k.band_items = ((k.M + br - 1) / br) * k.band_chunks;
+    const bool fits = k.BN >= 64 &&  // one lane per tile of the band for the flag wait: at most 129 tiles
+                      (int64_t)br * k.scm * ies < (1ll << 31) && (int64_t)br * k.sgm * oes < (1ll << 31);
+    // ... and when there is an item for every CU: with fewer, the tile walk has
+    // more loads in flight
+    rows = fits && (a->variant == 7 ||
+                    (a->variant == 0 && (int64_t)k.N * ies >= 16384 && k.band_items >= current_cu_count()));
+  }
+  ReduceFn fn = vec ? pick(k.c_dt, k.cg_dt, k.ws, a->variant, k.sys != 0, rows) : nullptr;
+  if (!fn) {
+    fn = &reduce_tiles_generic_kernel;
+    rows = false;
+  }
+  if (rows) {
+    grid = a->num_sms > 0 ? a->num_sms : 2 * current_cu_count();
+    if (grid > k.band_items) grid = k.band_items;
+  }
   hipLaunchKernelGGL(fn, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), k);
-  return hipGetLastError();
+  hipError_t err = hipGetLastError();
+  if (err == hipSuccess && rows && k.wait_flags && k.ws > 1) {
+    hipLaunchKernelGGL(reset_consumed_flags_kernel, dim3((k.total_tiles + 255) / 256), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), k.flags, k.ws - 1, k.total_tiles);
+    err = hipGetLastError();
+  }
+  return err;
 }
 
 extern "C" int iris_signal_tiles_launch(int32_t* tile_completed, const uint64_t* heap_bases, int32_t total_tiles,

@@ -25,7 +25,7 @@ def signal_all(shmem, flags, total, ws):
         ops.signal_tiles(shmem.on_rank(flags, r), shmem.get_heap_bases(), total, r, ws)
 
 
-@pytest.mark.parametrize("variant", range(0, 7))
+@pytest.mark.parametrize("variant", range(0, 9))  # 1-6: tile-kernel tuning points, 7: row bands, 8: tiles
 def test_eight_fp32_partials_to_bf16_is_bit_exact(shmem, variant):
     M, N, BM, BN, ws = 1024, 768, 256, 256, 8
     c = shmem.zeros((M, N), dtype=torch.float32)
@@ -56,7 +56,8 @@ def test_eight_fp32_partials_to_bf16_is_bit_exact(shmem, variant):
     (torch.float32, torch.bfloat16, 1, 128, 128, 64, 64, 0),    # one rank: plain cast, no flags
     (torch.float16, torch.bfloat16, 2, 64, 64, 64, 64, 0),      # no vector kernel for this pair
 ])
-def test_reduce_shapes_types_and_ragged_tiles(shmem, in_dt, out_dt, ws, M, N, BM, BN, grid):
+@pytest.mark.parametrize("variant", [0, 7])
+def test_reduce_shapes_types_and_ragged_tiles(shmem, in_dt, out_dt, ws, M, N, BM, BN, grid, variant):
     c = shmem.zeros((M, N), dtype=in_dt)
     cg = shmem.full((M, N), 3, dtype=out_dt)
     total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
@@ -64,13 +65,14 @@ def test_reduce_shapes_types_and_ragged_tiles(shmem, in_dt, out_dt, ws, M, N, BM
     host = fill_partials(shmem, c, ws, seed=M * 7 + N)
     signal_all(shmem, flags, total, ws)
     ops.one_shot_reduce(c, cg, flags, shmem.get_heap_bases(), 0, ws, BM, BN, 4, num_sms=grid,
-                        num_xcds=8 if grid == 256 else 1)
+                        num_xcds=8 if grid == 256 else 1, variant=variant)
     torch.cuda.synchronize()
     assert torch.equal(cg.cpu(), O.one_shot_reduce(host, out_dt))
     assert flags.cpu().tolist() == [0] * total
 
 
-def test_reduce_on_a_middle_rank_and_strided_buffers(shmem):
+@pytest.mark.parametrize("variant", [0, 7])
+def test_reduce_on_a_middle_rank_and_strided_buffers(shmem, variant):
     M, N, ws = 192, 160, 4
     wide = shmem.zeros((M, N + 32), dtype=torch.float32)
     c = wide[:, 16:16 + N]  # a view: row stride N+32, 64-byte column offset
@@ -87,7 +89,7 @@ def test_reduce_on_a_middle_rank_and_strided_buffers(shmem):
     signal_all(shmem, flags, total, ws)
     rank = 2
     ops.one_shot_reduce(shmem.on_rank(c, rank), shmem.on_rank(cg, rank), shmem.on_rank(flags, rank),
-                        shmem.get_heap_bases(), rank, ws, 64, 32, 2)
+                        shmem.get_heap_bases(), rank, ws, 64, 32, 2, variant=variant)
     torch.cuda.synchronize()
     assert torch.equal(shmem.on_rank(cg, rank).cpu(), O.one_shot_reduce(host, torch.bfloat16))
     assert float(shmem.on_rank(cg_wide, rank)[:, :8].float().abs().max()) == 0.0
@@ -95,7 +97,8 @@ def test_reduce_on_a_middle_rank_and_strided_buffers(shmem):
     assert flags.cpu().tolist() == [ws - 1] * total
 
 
-def test_only_signalled_tiles_are_reduced_and_the_wait_is_bounded(shmem):
+@pytest.mark.parametrize("variant", [0, 7])
+def test_only_signalled_tiles_are_reduced_and_the_wait_is_bounded(shmem, variant):
     """Flags gate tiles one by one: with every third tile signalled, exactly
     those tiles' regions (per the oracle's tile map) are written; the others
     time out, are reported and are left alone."""
@@ -111,7 +114,7 @@ def test_only_signalled_tiles_are_reduced_and_the_wait_is_bounded(shmem):
     flags.copy_(f)
     status = torch.zeros(1, dtype=torch.int32, device="cuda")
     ops.one_shot_reduce(c, cg, flags, shmem.get_heap_bases(), 0, ws, BM, BN, G, status=status,
-                        spin_timeout_ticks=1000)
+                        spin_timeout_ticks=1000, variant=variant)
     torch.cuda.synchronize()
     want = torch.full((M, N), -7.0)
     full = O.one_shot_reduce(host, torch.float32)
