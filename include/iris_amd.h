@@ -74,7 +74,7 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 #define IRIS_DTYPE_F32 0
 #define IRIS_DTYPE_F16 1
 #define IRIS_DTYPE_BF16 2
-/* integer element types: only iris_rma_selftest_launch takes them */
+/* integer element types: only iris_rma_selftest_launch and iris_p2p_bench_launch take them */
 #define IRIS_DTYPE_I8 3
 #define IRIS_DTYPE_I16 4
 #define IRIS_DTYPE_I32 5
@@ -263,6 +263,31 @@ int iris_mfma_probe_launch(const void* operands, float* sink, int32_t ab_dtype, 
 int iris_rma_selftest_launch(int32_t op, int32_t dtype, int32_t sem, int32_t scope, const void* data, void* results,
                              const uint64_t* heap_bases, int32_t cur_rank, int32_t num_ranks, int32_t block_size,
                              void* stream);
+
+/*
+ * The kernels of the reference's point-to-point microbenchmarks as HIP kernels
+ * over include/iris_device.hpp.  Thread i of a grid of ceil(n / block_size)
+ * blocks owns element i of `buffer` and `result`, both at the same heap offset
+ * on every rank; the launch acts as rank `cur_rank`.
+ *   LOAD        result[i] = load(buffer + i) from `peer_rank`          examples/00_load/load_bench.py:20-47
+ *   LOCAL_STORE result[i] = 0, the benchmarks' local baseline          examples/00_load/load_bench.py:50-61
+ *   STORE       store(buffer + i, i) on `peer_rank`                    examples/01_store/store_bench.py:18-45
+ *   ALL_LOAD    result[i] = sum over all ranks of load(buffer + i)     examples/02_all_load/all_load_bench.py:43-87
+ *   ALL_STORE   store(buffer + i, i) on every other rank               examples/03_all_store/all_store_bench.py:20-47
+ *   ATOMIC_ADD  atomic_add(buffer + i, 1) on `peer_rank`, relaxed, sys examples/04_atomic_add/atomic_add_bench.py:18-40
+ *   ATOMIC_XCHG result[i] = atomic_xchg(buffer + i, 1) on `peer_rank`  examples/05_atomic_xchg/atomic_xchg_bench.py:18-43
+ * dtype: F32, F16, BF16, I8 (no atomics), I32.  block_size is 1..1024.
+ */
+#define IRIS_P2P_LOAD 0
+#define IRIS_P2P_LOCAL_STORE 1
+#define IRIS_P2P_STORE 2
+#define IRIS_P2P_ALL_LOAD 3
+#define IRIS_P2P_ALL_STORE 4
+#define IRIS_P2P_ATOMIC_ADD 5
+#define IRIS_P2P_ATOMIC_XCHG 6
+int iris_p2p_bench_launch(int32_t op, int32_t dtype, void* buffer, void* result, int64_t n_elements,
+                          int32_t cur_rank, int32_t peer_rank, int32_t num_ranks, const uint64_t* heap_bases,
+                          int32_t block_size, void* stream);
 
 /* Library version, bumped when a signature in this header changes. */
 int iris_amd_abi_version(void);

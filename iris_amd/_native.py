@@ -139,6 +139,8 @@ SIGNATURES = {
     "iris_tile_map_host": (None, [ctypes.c_int32] * 6 + [ctypes.POINTER(ctypes.c_int32)] * 2),
     "iris_mfma_probe_launch": (_I, [_P, _P, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P]),
     "iris_rma_selftest_launch": (_I, [ctypes.c_int32] * 4 + [_P, _P, _P] + [ctypes.c_int32] * 3 + [_P]),
+    "iris_p2p_bench_launch": (_I, [ctypes.c_int32] * 2 + [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 3
+                              + [_P, ctypes.c_int32, _P]),
     "iris_amd_abi_version": (_I, []),
 }
 ALLOCATOR_SYMBOLS = ("finegrained_hipMalloc", "finegrained_hipFree")

@@ -375,6 +375,33 @@ def rma_selftest(op, data, results, heap_bases, rank, num_ranks, block_size, *, 
         _ptr(heap_bases), rank, num_ranks, block_size, ctypes.c_void_p(stream)))
 
 
+# iris_p2p_bench_launch (include/iris_amd.h)
+P2P_OPS = {"load": 0, "local_store": 1, "store": 2, "all_load": 3, "all_store": 4, "atomic_add": 5,
+           "atomic_xchg": 6}
+
+
+def p2p_bench(op, buffer, result, heap_bases, rank, peer, num_ranks, *, block_size=512):
+    """One launch of a point-to-point microbenchmark kernel as rank ``rank``:
+    ``op`` is a key of ``P2P_OPS`` (examples/00_load .. 05_atomic_xchg of the
+    reference); thread i owns element i of ``buffer`` / ``result``."""
+    ref = buffer if buffer is not None else result
+    if ref is None:
+        raise ValueError("a buffer is needed")
+    if ref.dtype not in _RMA_DTYPES or ref.dtype in (torch.int16, torch.int64):
+        raise ValueError(f"unsupported element type {ref.dtype}")
+    if buffer is not None and result is not None and (buffer.dtype != result.dtype or buffer.numel() != result.numel()):
+        raise ValueError("buffer and result must have the same element type and length")
+    if op != "local_store":
+        _check_heap_bases(heap_bases, num_ranks, ref.device)
+    stream = torch.cuda.current_stream(ref.device).cuda_stream
+    err = _native.lib().iris_p2p_bench_launch(
+        P2P_OPS[op], _RMA_DTYPES[ref.dtype], _ptr(buffer), _ptr(result), ref.numel(), rank, peer, num_ranks,
+        _ptr(heap_bases), block_size, ctypes.c_void_p(stream))
+    if err == _native.HIP_ERROR_INVALID_VALUE:
+        raise ValueError("iris_p2p_bench_launch rejected the arguments")
+    _native.hip_try(err)
+
+
 def signal_tiles(tile_completed, heap_bases, total_tiles, rank, world_size, *, include_self=False,
                  scope=SCOPE_AGENT):
     """+1 (release) on the flag of every tile on the other ranks (on every rank
