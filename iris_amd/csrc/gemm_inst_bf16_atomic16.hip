@@ -3,6 +3,8 @@
 
 namespace iris_amd {
 
+IRIS_GEMM_VARIANTS(IRIS_GEMM_INSTANTIATE, IRIS_DTYPE_BF16, OP_ATOMIC16)
+
 static const GemmKernelEntry k_entries[] = {IRIS_GEMM_VARIANTS(IRIS_GEMM_ENTRY, IRIS_DTYPE_BF16, OP_ATOMIC16)};
 
 const GemmKernelEntry* gemm_entries_bf16_atomic16(int* count) {

@@ -216,11 +216,25 @@ __device__ inline IRIS_GLOBAL P* rank_ptr(const GemmKArgs& p, P* ptr, int r) {
 template <class Cfg>
 struct Loader {
   __amdgpu_buffer_rsrc_t ra, rb;
-  uint32_t voff[Cfg::L];  // byte offset of (row, logical chunk) at k0 == 0
-  int kcol[Cfg::L];       // first k of the chunk at k0 == 0
-  int k_limit;            // K, or 0 once the program has no more steps to load
+  // Byte offset of (row, logical chunk) at k0 == 0 for each load, as the next
+  // step to be loaded needs it: chunks that lie past K in that step (only the
+  // K loop's last step can have them) are parked out of range and read as
+  // zero, the masked tail of gemm_*:186-195.  The masking is done once, when
+  // the load cursor reaches such a step, so that the K-steps themselves issue
+  // their loads without any vector arithmetic.
+  uint32_t voff[Cfg::L];
+  int k_limit;  // K
 
-  __device__ inline void setup(const GemmKArgs& p, const Item& it, int wave, int lane) {
+  // first k of the chunk that load `i` of this lane fetches at k0 == 0
+  __device__ static inline int chunk_k(int i, int wave, int lane) {
+    const bool isA = i < Cfg::A_LOADS;
+    const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
+    const int row = blk * Cfg::RPB + lane / Cfg::CPR;
+    return ((lane % Cfg::CPR) ^ ((row / Cfg::RP) % Cfg::CPR)) * 8;
+  }
+
+  // Offsets for the item's first step to be loaded, `k`.
+  __device__ inline void setup(const GemmKArgs& p, const Item& it, int wave, int lane, int k) {
     // Rows past the matrix edge re-read the last valid row (the reference
     // wraps with % M / % N, gemm_*:162-163); their results are never stored.
     const int m0c = min(it.m0, p.M - 1), n0c = min(it.n0, p.N - 1);
@@ -237,29 +251,38 @@ struct Loader {
       const bool isA = i < Cfg::A_LOADS;
       const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
       const int row = blk * Cfg::RPB + lane / Cfg::CPR;
-      const int ch = (lane % Cfg::CPR) ^ ((row / Cfg::RP) % Cfg::CPR);
       const int rclamp = min(row, (isA ? rows_a : rows_b) - 1);
       const int64_t ld = isA ? p.sam : p.sbn;
-      voff[i] = (uint32_t)(((int64_t)rclamp * ld + ch * 8) * 2);
-      kcol[i] = ch * 8;
-      if (p.debug & 2) voff[i] = (uint32_t)(ch * 16);
+      voff[i] = (uint32_t)(((int64_t)rclamp * ld + chunk_k(i, wave, lane)) * 2);
+      if (p.debug & 2) voff[i] = (uint32_t)(chunk_k(i, wave, lane) * 2);
     }
+    before_step(k, wave, lane);
+  }
+  // The load cursor is about to load step `k`: park the chunks past K.
+  __device__ inline void before_step(int k, int wave, int lane) {
+    if (k_limit - k * Cfg::BK >= Cfg::BK) return;  // a full step: nothing to mask
+#pragma unroll
+    for (int i = 0; i < Cfg::L; ++i)
+      if (k * Cfg::BK + chunk_k(i, wave, lane) >= k_limit) voff[i] = 0x80000000u;
+  }
+  // The program has no more steps to load: the loads are still issued, so
+  // that every K-step keeps the same number of loads in flight, but fetch
+  // nothing.
+  __device__ inline void park() {
+#pragma unroll
+    for (int i = 0; i < Cfg::L; ++i) voff[i] = 0x80000000u;
   }
 
-  // Issue load `i` of K-step `k` into the stage at LDS address `stage`.
-  // The K offset rides in the scalar offset; chunks past K read as zero: a
-  // vector offset beyond num_records is out of range for the buffer and the
-  // load returns 0 (the masked tail of gemm_*:186-195).  After the program's
-  // last step k_limit is 0: the loads are still issued, so that every K-step
-  // keeps the same number of loads in flight, but fetch nothing.
+  // Issue load `i` of K-step `k` into the stage at LDS address `stage`.  The
+  // K offset rides in the scalar offset.
   template <int I>
   __device__ inline void issue_one(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
     constexpr bool isA = I < Cfg::A_LOADS;
     const int k0 = k * Cfg::BK;
     const int blk = (isA ? I : I - Cfg::A_LOADS) * Cfg::NW + wave;
     IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + blk * 1024;
-    const uint32_t off = (k0 + kcol[I] < k_limit) ? voff[I] : 0x80000000u;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, (p.debug & 8) ? 0 : k0 * 2, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, voff[I],
+                                             (p.debug & 8) ? 0 : k0 * 2, 0, 0);
   }
   // the same with an index that is a constant once the caller's loop is unrolled
   __device__ inline void issue_at(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave, int i) const {
@@ -267,9 +290,8 @@ struct Loader {
     const int k0 = k * Cfg::BK;
     const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
     IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + blk * 1024;
-    const uint32_t off = (k0 + kcol[i] < k_limit) ? voff[i] : 0x80000000u;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, (p.debug & 8) ? 0 : k0 * 2, 0,
-                                             0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, voff[i],
+                                             (p.debug & 8) ? 0 : k0 * 2, 0, 0);
   }
   template <int I = 0>
   __device__ inline void issue(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
@@ -768,12 +790,14 @@ gemm_persistent_kernel(const GemmKArgs p) {
           const KRange kr = k_range<Cfg, SPLIT>(p, pid, l_item, nk);
           l_k = kr.k_begin;
           l_kend = kr.k_end;
-          ld.setup(p, l_it, wave, lane);
+          ld.setup(p, l_it, wave, lane, l_k);
         } else {
           l_k = 0;
           l_kend = nk;
-          ld.k_limit = 0;  // nothing left to load
+          ld.park();  // nothing left to load
         }
+      } else {
+        ld.before_step(l_k, wave, lane);
       }
     };
     Frags<Cfg> fr;
@@ -782,7 +806,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       const KRange kr = k_range<Cfg, SPLIT>(p, pid, 0, nk);
       l_k = kr.k_begin;
       l_kend = kr.k_end;
-      ld.setup(p, l_it, wave, lane);
+      ld.setup(p, l_it, wave, lane, l_k);
 #pragma unroll
       for (int s = 0; s < Cfg::S; ++s) {
         ld.issue(p, lds + s * Cfg::STAGE, l_k, wave);

@@ -42,25 +42,43 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 // The variants, in the launcher's order of preference: the first entry whose
 // compute tile divides the logical tile (and whose loader fits the operands)
 // wins.  `variant` k > 0 in iris_gemm_args forces entry k-1 (tuning runs).
-#define IRIS_GEMM_VARIANTS(X, DT, OP)                            \
-  X(DT, OP, 256, 256, 64, 2, 4, 2, true, "256x256x64_w2x4_s2")   \
-  X(DT, OP, 256, 128, 64, 2, 2, 2, true, "256x128x64_w2x2_s2")   \
-  X(DT, OP, 128, 256, 64, 1, 4, 2, true, "128x256x64_w1x4_s2")   \
-  X(DT, OP, 128, 128, 64, 2, 2, 4, true, "128x128x64_w2x2_s4")   \
-  X(DT, OP, 256, 64, 64, 4, 1, 2, true, "256x64x64_w4x1_s2")     \
-  X(DT, OP, 64, 64, 64, 2, 2, 4, true, "64x64x64_w2x2_s4")       \
-  X(DT, OP, 64, 64, 32, 2, 2, 1, false, "64x64x32_w2x2_generic")
+// Columns: compute tile CM, CN, BK; waves WM x WN; stages; LDS-DMA loader;
+// whether the tile also has a split-K build (must equal GemmCfg::SPLITK); name.
+#define IRIS_GEMM_VARIANTS(X, DT, OP)                               \
+  X(DT, OP, 256, 256, 64, 2, 4, 2, true, 0, "256x256x64_w2x4_s2")   \
+  X(DT, OP, 256, 128, 64, 2, 2, 2, true, 0, "256x128x64_w2x2_s2")   \
+  X(DT, OP, 128, 256, 64, 1, 4, 2, true, 0, "128x256x64_w1x4_s2")   \
+  X(DT, OP, 128, 128, 64, 2, 2, 4, true, 1, "128x128x64_w2x2_s4")   \
+  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 1, "256x64x64_w4x1_s2")     \
+  X(DT, OP, 64, 64, 64, 2, 2, 4, true, 1, "64x64x64_w2x2_s4")       \
+  X(DT, OP, 64, 64, 32, 2, 2, 1, false, 0, "64x64x32_w2x2_generic")
 
 // extra variants, compiled for the bf16 store op only (tuning runs, and the
 // one-substep stage whose fragment buffers alternate from step to step)
-#define IRIS_GEMM_TUNING_VARIANTS(X, DT, OP)                     \
-  X(DT, OP, 256, 128, 32, 2, 4, 4, true, "256x128x32_w2x4_s4")   \
-  X(DT, OP, 256, 128, 64, 2, 4, 2, true, "256x128x64_w2x4_s2")   \
-  X(DT, OP, 128, 256, 64, 2, 4, 2, true, "128x256x64_w2x4_s2")   \
-  X(DT, OP, 128, 128, 32, 2, 2, 4, true, "128x128x32_w2x2_s4")
+#define IRIS_GEMM_TUNING_VARIANTS(X, DT, OP)                        \
+  X(DT, OP, 256, 128, 32, 2, 4, 4, true, 0, "256x128x32_w2x4_s4")   \
+  X(DT, OP, 256, 128, 64, 2, 4, 2, true, 1, "256x128x64_w2x4_s2")   \
+  X(DT, OP, 128, 256, 64, 2, 4, 2, true, 1, "128x256x64_w2x4_s2")   \
+  X(DT, OP, 128, 128, 32, 2, 2, 4, true, 0, "128x128x32_w2x2_s4")
 
-#define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, NAME) \
+#define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, SPLIT, NAME) \
   make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP>(NAME),
+
+// Explicit instantiation of an entry's kernels.  Taking their addresses in
+// make_entry should be enough, but with the plain and the split-K build of a
+// tile in one translation unit the compiler's host pass has been seen to
+// reference one of the two without emitting it.
+#define IRIS_GEMM_ODT(DT, OP) (((OP) == OP_STORE32 || (OP) == OP_ATOMIC32) ? IRIS_DTYPE_F32 : (DT))
+#define IRIS_GEMM_INSTANTIATE_SPLIT_0(DT, OP, CM, CN, BK, WM, WN, S, DMA) \
+  static_assert(!GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>::SPLITK, "split-K column of the variant table");
+#define IRIS_GEMM_INSTANTIATE_SPLIT_1(DT, OP, CM, CN, BK, WM, WN, S, DMA)                                  \
+  static_assert(GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>::SPLITK, "split-K column of the variant table"); \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP,           \
+                                                  IRIS_GEMM_ODT(DT, OP), true>(const GemmKArgs);
+#define IRIS_GEMM_INSTANTIATE(DT, OP, CM, CN, BK, WM, WN, S, DMA, SPLIT, NAME)                    \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP,    \
+                                                  IRIS_GEMM_ODT(DT, OP), false>(const GemmKArgs); \
+  IRIS_GEMM_INSTANTIATE_SPLIT_##SPLIT(DT, OP, CM, CN, BK, WM, WN, S, DMA)
 
 #define IRIS_GEMM_DECLARE(TAG) const GemmKernelEntry* gemm_entries_##TAG(int* count);
 IRIS_GEMM_DECLARE(bf16_store16)
