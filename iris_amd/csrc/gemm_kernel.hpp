@@ -454,7 +454,10 @@ struct StoreCount {
   static constexpr int NV = 32 / (64 / Cfg::U16);
   static constexpr int FAST_STORES = (Cfg::TM / 32) * NPASS * NV;
 };
-template <class Cfg, int OP, int ODT>
+// WSB: 0 when the wave's 32 scratch rows are contiguous; otherwise the scratch
+// is made of 1 KiB pieces WSB bytes apart (the ring-of-five kernel lends the
+// epilogue the parts of a free slab slot that the wave itself refills).
+template <class Cfg, int OP, int ODT, int WSB = 0>
 __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM][Cfg::IN], IRIS_LDS char* ws,
                                  int wm0, int wn0, int m_end, int n_end, int lane) {  // lane: by value, see below
   constexpr bool F32 = (OP == OP_STORE32 || OP == OP_ATOMIC32);
@@ -463,6 +466,10 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
   constexpr int NPASS = Cfg::TN / CP;     // 1 (16-bit) or 2 (fp32)
   constexpr int NJ = CP / 16;             // 16-column accumulator blocks per pass
   constexpr int EPV = 16 / ES;            // elements per 16-byte unit
+  constexpr int RPK = 1024 / Cfg::WS_PITCH;  // scratch rows per KiB
+  auto srow = [](int row) __attribute__((always_inline)) {
+    return WSB == 0 ? row * Cfg::WS_PITCH : (row / RPK) * WSB + (row % RPK) * Cfg::WS_PITCH;
+  };
   // Everything below depends on the lane id.  It is made opaque here so that
   // the address arithmetic of the epilogue is computed in the epilogue and
   // not hoisted into registers that stay live across the K loop.
@@ -491,11 +498,11 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
             const f32x4 a4 = acc[i * 2 + ib][ps * NJ + g];
             if constexpr (F32) {
               const int u = (g * 4 + lq) ^ sw;
-              *reinterpret_cast<IRIS_LDS f32x4*>(ws + row * Cfg::WS_PITCH + u * 16) = a4;
+              *reinterpret_cast<IRIS_LDS f32x4*>(ws + srow(row) + u * 16) = a4;
             } else {
               const int u = (g * 2 + (lq >> 1)) ^ sw;
               const u32x2 v = {pack2<ODT>(a4[0], a4[1]), pack2<ODT>(a4[2], a4[3])};
-              *reinterpret_cast<IRIS_LDS u32x2*>(ws + row * Cfg::WS_PITCH + u * 16 + (lq & 1) * 8) = v;
+              *reinterpret_cast<IRIS_LDS u32x2*>(ws + srow(row) + u * 16 + (lq & 1) * 8) = v;
             }
           }
         }
@@ -520,7 +527,7 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
               const int row = idx / CP, cc = idx % CP;
               const int u = (cc / 4) ^ ((row / Cfg::ERPB) % Cfg::U16);
               const float v =
-                  *reinterpret_cast<const IRIS_LDS float*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 4) * 4);
+                  *reinterpret_cast<const IRIS_LDS float*>(ws + srow(row) + u * 16 + (cc % 4) * 4);
               const int m = row0 + row, n = col0 + cc;
               if (m < m_end && n < n_end)
                 __hip_atomic_fetch_add((IRIS_GLOBAL float*)(dst + ((int64_t)m * p.som + (int64_t)n * p.son) * 4),
@@ -536,7 +543,7 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
                 const int row = idx / (CP / 2), cc = (idx % (CP / 2)) * 2;
                 const int u = (cc / 8) ^ ((row / Cfg::ERPB) % Cfg::U16);
                 const unsigned int v =
-                    *reinterpret_cast<const IRIS_LDS unsigned int*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 8) * 2);
+                    *reinterpret_cast<const IRIS_LDS unsigned int*>(ws + srow(row) + u * 16 + (cc % 8) * 2);
                 const int m = row0 + row, n = col0 + cc;
                 atomic_add16_pair<ODT>((IRIS_GLOBAL unsigned int*)(dst + ((int64_t)m * p.som + n) * 2), v);
               }
@@ -555,7 +562,7 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
                 const int row = t * RPI + lane / Cfg::U16;
                 const int u = lane % Cfg::U16;
                 const int pu = u ^ ((row / Cfg::ERPB) % Cfg::U16);
-                v[t] = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + row * Cfg::WS_PITCH + pu * 16);
+                v[t] = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + srow(row) + pu * 16);
                 off[t] = (u + 1) * EPV <= cols_ok ? (int)((row * p.som + u * EPV) * ES) : (int)0x80000000;
               }
 #pragma unroll
@@ -567,7 +574,7 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
             for (int idx = lane; idx < 32 * CP; idx += 64) {
               const int row = idx / CP, cc = idx % CP;
               const int u = (cc / EPV) ^ ((row / Cfg::ERPB) % Cfg::U16);
-              const IRIS_LDS char* src = ws + row * Cfg::WS_PITCH + u * 16 + (cc % EPV) * ES;
+              const IRIS_LDS char* src = ws + srow(row) + u * 16 + (cc % EPV) * ES;
               const int m = row0 + row, n = col0 + cc;
               if (m < m_end && n < n_end) {
                 IRIS_GLOBAL char* d = dst + ((int64_t)m * p.som + (int64_t)n * p.son) * ES;

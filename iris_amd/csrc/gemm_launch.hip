@@ -149,6 +149,9 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   auto fits = [&](const GemmKernelEntry& e) {
     if (!e.dma) return true;
     if (!dma_ok) return false;
+    // ring of five: whole 64-k steps, one compute tile per logical tile
+    if (e.ring5 && (a.K < 64 || a.K % 64 != 0 || a.block_m != e.cm || a.block_n != e.cn || a.split_k > 1))
+      return false;
     const int64_t lim = (int64_t)1 << 31;
     return ((int64_t)e.cm * a.stride_am + a.K) * 2 < lim && ((int64_t)e.cn * a.stride_bn + a.K) * 2 < lim;
   };
@@ -164,7 +167,7 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
     // columns a small matrix cannot fill are not worth a tall compute tile
     for (int i = 0; i < count && !pick; ++i) {
       const GemmKernelEntry& e = list[i];
-      if (!fits(e)) continue;
+      if (e.ring5 || !fits(e)) continue;
       if (a.block_m % e.cm != 0 || a.block_n % e.cn != 0) continue;
       if (e.cm > 64 && e.cm >= 2 * a.M) continue;
       if (e.cn > 64 && e.cn >= 2 * a.N) continue;
