@@ -4,9 +4,8 @@
 namespace iris_amd {
 
 IRIS_GEMM_VARIANTS(IRIS_GEMM_INSTANTIATE, IRIS_DTYPE_F16, OP_STORE32)
-IRIS_GEMM_RING5_INSTANTIATE(IRIS_DTYPE_F16, OP_STORE32)
 
-static const GemmKernelEntry k_entries[] = {IRIS_GEMM_VARIANTS(IRIS_GEMM_ENTRY, IRIS_DTYPE_F16, OP_STORE32) make_ring5_entry<IRIS_DTYPE_F16, OP_STORE32>()};
+static const GemmKernelEntry k_entries[] = {IRIS_GEMM_VARIANTS(IRIS_GEMM_ENTRY, IRIS_DTYPE_F16, OP_STORE32)};
 
 const GemmKernelEntry* gemm_entries_f16_store32(int* count) {
   *count = (int)(sizeof(k_entries) / sizeof(k_entries[0]));

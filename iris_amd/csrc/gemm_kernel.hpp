@@ -70,7 +70,6 @@ struct GemmKArgs {
   int64_t partial_stride;
   uint32_t* status;   // optional: IRIS_STATUS_SPIN_TIMEOUT when a wait for a partial gave up
   uint64_t timeout;   // bound of that wait, 100 MHz ticks
-  int debug;         // tuning experiments only (IRIS_AMD_GEMM_DEBUG): 1 = fetch nothing, 2 = every row fetches row 0, 4 = store nothing
 };
 
 template <int DT>
@@ -216,87 +215,71 @@ __device__ inline IRIS_GLOBAL P* rank_ptr(const GemmKArgs& p, P* ptr, int r) {
 template <class Cfg>
 struct Loader {
   __amdgpu_buffer_rsrc_t ra, rb;
-  // Byte offset of (row, logical chunk) at k0 == 0 for each load, as the next
-  // step to be loaded needs it: chunks that lie past K in that step (only the
-  // K loop's last step can have them) are parked out of range and read as
-  // zero, the masked tail of gemm_*:186-195.  The masking is done once, when
-  // the load cursor reaches such a step, so that the K-steps themselves issue
-  // their loads without any vector arithmetic.
-  uint32_t voff[Cfg::L];
+  // Byte offset, at k0 == 0, of the 16-byte chunk this lane fetches with the
+  // first A load and the first B load of a slab; load i of an operand is
+  // i * NW * RPB rows further down (step_a / step_b bytes).  Rows below the
+  // matrix edge lie past the end of the buffer descriptor and read as zero.
+  // For the one K-step that can hold chunks past K, the K loop's last, the
+  // offsets of those lanes are parked out of range when the load cursor
+  // reaches the step (the masked tail of gemm_*:186-195), so the K-steps
+  // issue their loads without any per-load arithmetic but one add.
+  uint32_t va, vb;
+  int step_a, step_b;
   int k_limit;  // K
 
-  // first k of the chunk that load `i` of this lane fetches at k0 == 0
-  __device__ static inline int chunk_k(int i, int wave, int lane) {
-    const bool isA = i < Cfg::A_LOADS;
-    const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
-    const int row = blk * Cfg::RPB + lane / Cfg::CPR;
+  // The chunk of the row that a lane fetches is the same for every load:
+  // the swizzle period divides the rows between two loads of a wave.
+  static_assert((Cfg::NW * Cfg::RPB / Cfg::RP) % Cfg::CPR == 0, "the lane's chunk must not depend on the load");
+  // first k of the chunk that this lane fetches at k0 == 0
+  __device__ static inline int chunk_k(int wave, int lane) {
+    const int row = wave * Cfg::RPB + lane / Cfg::CPR;
     return ((lane % Cfg::CPR) ^ ((row / Cfg::RP) % Cfg::CPR)) * 8;
   }
 
   // Offsets for the item's first step to be loaded, `k`.
   __device__ inline void setup(const GemmKArgs& p, const Item& it, int wave, int lane, int k) {
-    // Rows past the matrix edge re-read the last valid row (the reference
-    // wraps with % M / % N, gemm_*:162-163); their results are never stored.
+    // a tile that starts past the matrix edge (a masked sub-tile) reads nothing
     const int m0c = min(it.m0, p.M - 1), n0c = min(it.n0, p.N - 1);
-    const int rows_a = min(Cfg::CM, p.M - m0c), rows_b = min(Cfg::CN, p.N - n0c);
+    const int rows_a = it.m0 < p.M ? min(Cfg::CM, p.M - it.m0) : 0, rows_b = it.n0 < p.N ? min(Cfg::CN, p.N - it.n0) : 0;
     const char* abase = p.a + (int64_t)m0c * p.sam * 2;
     const char* bbase = p.b + (int64_t)n0c * p.sbn * 2;
-    const uint32_t arec = (uint32_t)(((int64_t)(rows_a - 1) * p.sam + p.K) * 2);
-    const uint32_t brec = (uint32_t)(((int64_t)(rows_b - 1) * p.sbn + p.K) * 2);
+    const uint32_t arec = rows_a > 0 ? (uint32_t)(((int64_t)(rows_a - 1) * p.sam + p.K) * 2) : 0;
+    const uint32_t brec = rows_b > 0 ? (uint32_t)(((int64_t)(rows_b - 1) * p.sbn + p.K) * 2) : 0;
     ra = __builtin_amdgcn_make_buffer_rsrc((void*)abase, 0, arec, 0x00020000);
     rb = __builtin_amdgcn_make_buffer_rsrc((void*)bbase, 0, brec, 0x00020000);
-    k_limit = (p.debug & 1) ? 0 : p.K;
-#pragma unroll
-    for (int i = 0; i < Cfg::L; ++i) {
-      const bool isA = i < Cfg::A_LOADS;
-      const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
-      const int row = blk * Cfg::RPB + lane / Cfg::CPR;
-      const int rclamp = min(row, (isA ? rows_a : rows_b) - 1);
-      const int64_t ld = isA ? p.sam : p.sbn;
-      voff[i] = (uint32_t)(((int64_t)rclamp * ld + chunk_k(i, wave, lane)) * 2);
-      if (p.debug & 2) voff[i] = (uint32_t)(chunk_k(i, wave, lane) * 2);
-    }
+    k_limit = p.K;
+    const int row = wave * Cfg::RPB + lane / Cfg::CPR, ck = chunk_k(wave, lane);
+    va = (uint32_t)(((int64_t)row * p.sam + ck) * 2);
+    vb = (uint32_t)(((int64_t)row * p.sbn + ck) * 2);
+    step_a = (int)((int64_t)Cfg::NW * Cfg::RPB * p.sam * 2);
+    step_b = (int)((int64_t)Cfg::NW * Cfg::RPB * p.sbn * 2);
     before_step(k, wave, lane);
   }
   // The load cursor is about to load step `k`: park the chunks past K.
   __device__ inline void before_step(int k, int wave, int lane) {
     if (k_limit - k * Cfg::BK >= Cfg::BK) return;  // a full step: nothing to mask
-#pragma unroll
-    for (int i = 0; i < Cfg::L; ++i)
-      if (k * Cfg::BK + chunk_k(i, wave, lane) >= k_limit) voff[i] = 0x80000000u;
+    if (k * Cfg::BK + chunk_k(wave, lane) >= k_limit) va = vb = 0x80000000u;
   }
   // The program has no more steps to load: the loads are still issued, so
   // that every K-step keeps the same number of loads in flight, but fetch
   // nothing.
-  __device__ inline void park() {
-#pragma unroll
-    for (int i = 0; i < Cfg::L; ++i) voff[i] = 0x80000000u;
-  }
+  __device__ inline void park() { va = vb = 0x80000000u; }
 
   // Issue load `i` of K-step `k` into the stage at LDS address `stage`.  The
   // K offset rides in the scalar offset.
-  template <int I>
-  __device__ inline void issue_one(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
-    constexpr bool isA = I < Cfg::A_LOADS;
-    const int k0 = k * Cfg::BK;
-    const int blk = (isA ? I : I - Cfg::A_LOADS) * Cfg::NW + wave;
-    IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + blk * 1024;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, voff[I],
-                                             (p.debug & 8) ? 0 : k0 * 2, 0, 0);
-  }
-  // the same with an index that is a constant once the caller's loop is unrolled
   __device__ inline void issue_at(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave, int i) const {
     const bool isA = i < Cfg::A_LOADS;
+    const int j = isA ? i : i - Cfg::A_LOADS;
     const int k0 = k * Cfg::BK;
-    const int blk = (isA ? i : i - Cfg::A_LOADS) * Cfg::NW + wave;
-    IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + blk * 1024;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, voff[i],
-                                             (p.debug & 8) ? 0 : k0 * 2, 0, 0);
+    IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + (j * Cfg::NW + wave) * 1024;
+    // (a parked offset stays out of range: j * step is far below 2 GiB)
+    const uint32_t off = isA ? va + (uint32_t)(j * step_a) : vb + (uint32_t)(j * step_b);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, k0 * 2, 0, 0);
   }
   template <int I = 0>
   __device__ inline void issue(const GemmKArgs& p, IRIS_LDS char* stage, int k, int wave) const {
     if constexpr (I < Cfg::L) {
-      issue_one<I>(p, stage, k, wave);
+      issue_at(p, stage, k, wave, I);
       issue<I + 1>(p, stage, k, wave);
     }
   }
@@ -454,10 +437,7 @@ struct StoreCount {
   static constexpr int NV = 32 / (64 / Cfg::U16);
   static constexpr int FAST_STORES = (Cfg::TM / 32) * NPASS * NV;
 };
-// WSB: 0 when the wave's 32 scratch rows are contiguous; otherwise the scratch
-// is made of 1 KiB pieces WSB bytes apart (the ring-of-five kernel lends the
-// epilogue the parts of a free slab slot that the wave itself refills).
-template <class Cfg, int OP, int ODT, int WSB = 0>
+template <class Cfg, int OP, int ODT>
 __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM][Cfg::IN], IRIS_LDS char* ws,
                                  int wm0, int wn0, int m_end, int n_end, int lane) {  // lane: by value, see below
   constexpr bool F32 = (OP == OP_STORE32 || OP == OP_ATOMIC32);
@@ -466,10 +446,6 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
   constexpr int NPASS = Cfg::TN / CP;     // 1 (16-bit) or 2 (fp32)
   constexpr int NJ = CP / 16;             // 16-column accumulator blocks per pass
   constexpr int EPV = 16 / ES;            // elements per 16-byte unit
-  constexpr int RPK = 1024 / Cfg::WS_PITCH;  // scratch rows per KiB
-  auto srow = [](int row) __attribute__((always_inline)) {
-    return WSB == 0 ? row * Cfg::WS_PITCH : (row / RPK) * WSB + (row % RPK) * Cfg::WS_PITCH;
-  };
   // Everything below depends on the lane id.  It is made opaque here so that
   // the address arithmetic of the epilogue is computed in the epilogue and
   // not hoisted into registers that stay live across the K loop.
@@ -498,11 +474,11 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
             const f32x4 a4 = acc[i * 2 + ib][ps * NJ + g];
             if constexpr (F32) {
               const int u = (g * 4 + lq) ^ sw;
-              *reinterpret_cast<IRIS_LDS f32x4*>(ws + srow(row) + u * 16) = a4;
+              *reinterpret_cast<IRIS_LDS f32x4*>(ws + row * Cfg::WS_PITCH + u * 16) = a4;
             } else {
               const int u = (g * 2 + (lq >> 1)) ^ sw;
               const u32x2 v = {pack2<ODT>(a4[0], a4[1]), pack2<ODT>(a4[2], a4[3])};
-              *reinterpret_cast<IRIS_LDS u32x2*>(ws + srow(row) + u * 16 + (lq & 1) * 8) = v;
+              *reinterpret_cast<IRIS_LDS u32x2*>(ws + row * Cfg::WS_PITCH + u * 16 + (lq & 1) * 8) = v;
             }
           }
         }
@@ -527,7 +503,7 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
               const int row = idx / CP, cc = idx % CP;
               const int u = (cc / 4) ^ ((row / Cfg::ERPB) % Cfg::U16);
               const float v =
-                  *reinterpret_cast<const IRIS_LDS float*>(ws + srow(row) + u * 16 + (cc % 4) * 4);
+                  *reinterpret_cast<const IRIS_LDS float*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 4) * 4);
               const int m = row0 + row, n = col0 + cc;
               if (m < m_end && n < n_end)
                 __hip_atomic_fetch_add((IRIS_GLOBAL float*)(dst + ((int64_t)m * p.som + (int64_t)n * p.son) * 4),
@@ -543,7 +519,7 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
                 const int row = idx / (CP / 2), cc = (idx % (CP / 2)) * 2;
                 const int u = (cc / 8) ^ ((row / Cfg::ERPB) % Cfg::U16);
                 const unsigned int v =
-                    *reinterpret_cast<const IRIS_LDS unsigned int*>(ws + srow(row) + u * 16 + (cc % 8) * 2);
+                    *reinterpret_cast<const IRIS_LDS unsigned int*>(ws + row * Cfg::WS_PITCH + u * 16 + (cc % 8) * 2);
                 const int m = row0 + row, n = col0 + cc;
                 atomic_add16_pair<ODT>((IRIS_GLOBAL unsigned int*)(dst + ((int64_t)m * p.som + n) * 2), v);
               }
@@ -562,7 +538,7 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
                 const int row = t * RPI + lane / Cfg::U16;
                 const int u = lane % Cfg::U16;
                 const int pu = u ^ ((row / Cfg::ERPB) % Cfg::U16);
-                v[t] = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + srow(row) + pu * 16);
+                v[t] = *reinterpret_cast<const IRIS_LDS u32x4*>(ws + row * Cfg::WS_PITCH + pu * 16);
                 off[t] = (u + 1) * EPV <= cols_ok ? (int)((row * p.som + u * EPV) * ES) : (int)0x80000000;
               }
 #pragma unroll
@@ -574,7 +550,7 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
             for (int idx = lane; idx < 32 * CP; idx += 64) {
               const int row = idx / CP, cc = idx % CP;
               const int u = (cc / EPV) ^ ((row / Cfg::ERPB) % Cfg::U16);
-              const IRIS_LDS char* src = ws + srow(row) + u * 16 + (cc % EPV) * ES;
+              const IRIS_LDS char* src = ws + row * Cfg::WS_PITCH + u * 16 + (cc % EPV) * ES;
               const int m = row0 + row, n = col0 + cc;
               if (m < m_end && n < n_end) {
                 IRIS_GLOBAL char* d = dst + ((int64_t)m * p.som + (int64_t)n * p.son) * ES;
@@ -750,15 +726,13 @@ gemm_persistent_kernel(const GemmKArgs p) {
         for (int q = 1; q < p.split_k; q += GROUP) add_partials<Cfg, GROUP>(p, acc, kr.slot, q, tid);
       }
     }
-    bool fast = false;
-    if (!(p.debug & 4))
-      fast = store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end,
-                                     c_it.n_end, lane);
+    const bool fast = store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN,
+                                              c_it.m_end, c_it.n_end, lane);
     if (c_it.last_sub) {
       if (defer_publish) {
         pending_tile = __builtin_amdgcn_readfirstlane(c_it.tile_id);
         // the count only holds for a tile that is a single compute tile
-        pending_skip = (fast && c_it.first_sub && !(p.debug & 64)) ? 1 : 0;
+        pending_skip = (fast && c_it.first_sub) ? 1 : 0;
       } else if (p.flag_mode != 0) {
         IRIS_WAIT_VMCNT(0);  // this wave's stores of the tile have completed
         __syncthreads();

@@ -132,10 +132,6 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   k.total_tiles = k.num_pid_m * k.num_pid_n;
   k.sys = a.scope == IRIS_SCOPE_SYSTEM;
   k.vec_out = vec_ok(k.out, k.som, k.son, dtype_size(out_dt)) ? 1 : 0;
-  {
-    static const int dbgflags = std::getenv("IRIS_AMD_GEMM_DEBUG") ? std::atoi(std::getenv("IRIS_AMD_GEMM_DEBUG")) : 0;
-    k.debug = dbgflags;
-  }
 
   int count = 0;
   const GemmKernelEntry* list = entries_for(a.ab_dtype, op, &count);
@@ -149,9 +145,6 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   auto fits = [&](const GemmKernelEntry& e) {
     if (!e.dma) return true;
     if (!dma_ok) return false;
-    // ring of five: whole 64-k steps, one compute tile per logical tile
-    if (e.ring5 && (a.K < 64 || a.K % 64 != 0 || a.block_m != e.cm || a.block_n != e.cn || a.split_k > 1))
-      return false;
     const int64_t lim = (int64_t)1 << 31;
     return ((int64_t)e.cm * a.stride_am + a.K) * 2 < lim && ((int64_t)e.cn * a.stride_bn + a.K) * 2 < lim;
   };
@@ -167,7 +160,7 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
     // columns a small matrix cannot fill are not worth a tall compute tile
     for (int i = 0; i < count && !pick; ++i) {
       const GemmKernelEntry& e = list[i];
-      if (e.ring5 || !fits(e)) continue;
+      if (!fits(e)) continue;
       if (a.block_m % e.cm != 0 || a.block_n % e.cn != 0) continue;
       if (e.cm > 64 && e.cm >= 2 * a.M) continue;
       if (e.cn > 64 && e.cn >= 2 * a.N) continue;

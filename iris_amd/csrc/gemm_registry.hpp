@@ -4,7 +4,6 @@
 #pragma once
 
 #include "gemm_kernel.hpp"
-#include "gemm_ring5.hpp"
 
 namespace iris_amd {
 
@@ -17,7 +16,6 @@ struct GemmKernelEntry {
   int bk, wm, wn, stages;
   bool dma;    // LDS-DMA loader (needs K-contiguous, 16-byte aligned operands)
   bool splitk;  // the kernel can share a tile's K range with other programs
-  bool ring5;   // gemm_ring5_kernel: five 32-k slabs in LDS, register epilogue (store ops, K % 64 == 0)
   int threads;
   int lds_bytes;
   GemmKernelFn fn;
@@ -37,21 +35,9 @@ template <class Cfg, int OP>
 constexpr GemmKernelEntry make_entry(const char* name) {
   constexpr int ODT = (OP == OP_STORE32 || OP == OP_ATOMIC32) ? IRIS_DTYPE_F32 : Cfg::DT;
   return GemmKernelEntry{Cfg::DT, OP,      Cfg::CM, Cfg::CN, Cfg::BK,        Cfg::WM,
-                         Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, false, Cfg::NT, Cfg::LDS_BYTES,
+                         Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::NT, Cfg::LDS_BYTES,
                          &gemm_persistent_kernel<Cfg, OP, ODT, false>, split_fn<Cfg, OP, ODT>(), name};
 }
-
-// the ring-of-five kernel of a store op, always the last entry of its list
-template <int DT, int OP>
-constexpr GemmKernelEntry make_ring5_entry() {
-  constexpr int ODT = OP == OP_STORE32 ? IRIS_DTYPE_F32 : DT;
-  using Cfg = Ring5Cfg<DT>;
-  return GemmKernelEntry{DT, OP, Cfg::CM, Cfg::CN, 64, Cfg::WM, Cfg::WN, RING5_SLOTS, true, false, true,
-                         Cfg::NT, ring5_lds_bytes<DT>(), &gemm_ring5_kernel<DT, OP, ODT>, nullptr,
-                         "256x256x64_w2x4_ring5"};
-}
-#define IRIS_GEMM_RING5_INSTANTIATE(DT, OP) \
-  template __global__ void gemm_ring5_kernel<DT, OP, IRIS_GEMM_ODT(DT, OP)>(const GemmKArgs);
 
 // The variants, in the launcher's order of preference: the first entry whose
 // compute tile divides the logical tile (and whose loader fits the operands)

@@ -196,8 +196,6 @@ def test_every_tuning_variant_is_correct(shmem, variant):
     if name is None:
         assert variant > 7  # the seven base tiles always exist
         pytest.skip("no such variant")
-    if "ring5" in name:
-        pytest.skip("whole 64-k steps only: covered by test_ring_of_five_kernel")
     dtype = torch.bfloat16
     M, N, K = 520, 776, 328
     A, B = make_ab(M, N, K, dtype, lda=336, ldb=344)
@@ -209,101 +207,6 @@ def test_every_tuning_variant_is_correct(shmem, variant):
     torch.cuda.synchronize()
     check_close(cg, O.shard_gemm(A, B, dtype), name)
     assert flags.cpu().tolist() == [1] * total
-
-
-def ring5_variant(dtype, out_f32):
-    for v in range(1, 40):
-        name = ops.gemm_variant_name(dtype, out_f32, False, v)
-        if name is None:
-            break
-        if "ring5" in name:
-            return v
-    raise AssertionError("the ring-of-five kernel is not in the list")
-
-
-@pytest.mark.parametrize("M,N,K,dtype,out_dtype,grid,lda", [
-    (256, 256, 64, torch.bfloat16, torch.bfloat16, 4, None),      # one tile, one step
-    (512, 768, 128, torch.bfloat16, torch.bfloat16, 8, None),     # two steps: the ring wraps inside a tile
-    (1024, 1280, 320, torch.bfloat16, torch.bfloat16, 8, 8192),   # five steps, several tiles a program, K-shard view
-    (300, 520, 64, torch.bfloat16, torch.bfloat16, 3, None),      # ragged M and N
-    (300, 516, 192, torch.float16, torch.float16, 256, None),     # N not a multiple of 8: element-wise stores
-    (768, 512, 256, torch.bfloat16, torch.float32, 5, None),      # fp32 destination
-])
-def test_ring_of_five_kernel(shmem, M, N, K, dtype, out_dtype, grid, lda):
-    """The five-slab kernel, forced: same results and flags as the oracle's shard GEMM."""
-    A, B = make_ab(M, N, K, dtype, lda=lda, ldb=lda)
-    a, b = to_heap(shmem, A), to_heap(shmem, B)
-    cg = shmem.full((M, N), -5, dtype=out_dtype)
-    total = ops.cdiv(M, 256) * ops.cdiv(N, 256)
-    flags = shmem.zeros((total,), dtype=torch.int32)
-    v = ring5_variant(dtype, out_dtype == torch.float32)
-    ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, grid, 256, 256, 64, 4, ops.EPI_ALL_SCATTER,
-                    num_xcds=8 if grid % 8 == 0 else 1, variant=v)
-    torch.cuda.synchronize()
-    check_close(cg, O.shard_gemm(A, B, None if out_dtype == torch.float32 else dtype))
-    assert flags.cpu().tolist() == [1] * total
-
-
-def test_ring_of_five_kernel_virtual_ranks_and_one_shot(shmem):
-    """All-scatter to 4 ranks and the one-shot producer/consumer pair through the five-slab kernel."""
-    ws, M, N, K = 4, 512, 512, 128
-    dtype = torch.bfloat16
-    hb = shmem.get_heap_bases()
-    v = ring5_variant(dtype, False)
-    # all-scatter: rank r's N-shard lands at column r*N of every rank's buffer
-    A, B = make_ab(M, N * ws, K, dtype)
-    a, b_full = to_heap(shmem, A), to_heap(shmem, B)
-    cg = shmem.zeros((M, N * ws), dtype=dtype)
-    total = ops.cdiv(M, 256) * ops.cdiv(N, 256)
-    flags = shmem.zeros((total,), dtype=torch.int32)
-    for r in range(ws):
-        shmem.on_rank(cg, r).zero_()
-        shmem.on_rank(flags, r).zero_()
-    for r in range(ws):
-        ops.gemm_launch(a, b_full[:, r * N:(r + 1) * N], None, shmem.on_rank(cg, r), shmem.on_rank(flags, r), hb, r, ws,
-                        8, 256, 256, 64, 4, ops.EPI_ALL_SCATTER, variant=v)
-    torch.cuda.synchronize()
-    want = O.shard_gemm(A, B, dtype)
-    for r in range(ws):
-        check_close(shmem.on_rank(cg, r), want, f"rank {r}")
-        assert shmem.on_rank(flags, r).cpu().tolist() == [ws] * total
-    # one-shot: fp32 partials, flags to the other ranks, reduce
-    A, B = make_ab(M, N, K * ws, dtype, scale=0.05)
-    a_full, b_full = to_heap(shmem, A), to_heap(shmem, B)
-    c = shmem.zeros((M, N), dtype=torch.float32)
-    out = shmem.zeros((M, N), dtype=dtype)
-    flags = shmem.zeros((total,), dtype=torch.int32)
-    for r in range(ws):
-        for t in (c, out, flags):
-            shmem.on_rank(t, r).zero_()
-    v32 = ring5_variant(dtype, True)  # the partials are fp32: the producer is a kernel of the fp32-store list
-    for phase in (ops.PHASE_PRODUCE, ops.PHASE_CONSUME):
-        for r in range(ws):
-            ops.gemm_launch(a_full[:, r * K:(r + 1) * K], b_full[r * K:(r + 1) * K, :], shmem.on_rank(c, r),
-                            shmem.on_rank(out, r), shmem.on_rank(flags, r), hb, r, ws, 8, 256, 256, 64, 6,
-                            ops.EPI_ONE_SHOT, phase=phase, variant=v32)
-        torch.cuda.synchronize()
-        if phase == ops.PHASE_PRODUCE:
-            for r in range(ws):
-                assert shmem.on_rank(flags, r).cpu().tolist() == [ws - 1] * total
-    partials = torch.stack([shmem.on_rank(c, r).cpu() for r in range(ws)])
-    for r in range(ws):
-        assert torch.equal(shmem.on_rank(out, r).cpu(), O.one_shot_reduce(partials, dtype))
-        assert shmem.on_rank(flags, r).cpu().tolist() == [0] * total
-    check_close(out, O.one_shot_all_reduce(O.k_shards(A, B, ws), torch.float32, dtype), "vs closed form")
-
-
-def test_ring_of_five_kernel_is_refused_where_it_does_not_fit(shmem):
-    A, B = make_ab(256, 256, 96, torch.bfloat16)
-    a, b = to_heap(shmem, A), to_heap(shmem, B)
-    cg = shmem.zeros((256, 256), dtype=torch.bfloat16)
-    v = ring5_variant(torch.bfloat16, False)
-    with pytest.raises(ValueError):   # K is not a multiple of 64
-        ops.gemm_launch(a, b, None, cg, None, None, 0, 1, 4, 256, 256, 64, 4, ops.EPI_ALL_SCATTER, variant=v)
-    A, B = make_ab(256, 256, 128, torch.bfloat16)
-    a, b = to_heap(shmem, A), to_heap(shmem, B)
-    with pytest.raises(ValueError):   # the logical tile is not 256 x 256
-        ops.gemm_launch(a, b, None, cg, None, None, 0, 1, 4, 128, 256, 64, 4, ops.EPI_ALL_SCATTER, variant=v)
 
 
 # --------------------------------------------------------------------------- atomics
