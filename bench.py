@@ -332,10 +332,17 @@ def run_decoder(args):
                                            shmem.on_rank(flags_dn, rank), hb, rank, ws, grid_dn, bm, bn, 64, 6,
                                            ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks),
                   "reduce": 1}
+            kern = {"gate_up": ops.gemm_plan_name(x, wg.T, None, shmem.on_rank(gate_all, rank),
+                                                  shmem.on_rank(flags_up, rank), hb, rank, ws, grid_up, bm, bn, 64, 4,
+                                                  ops.EPI_ALL_SCATTER, partials=P, locks=locks),
+                    "down": ops.gemm_plan_name(h, wd.T, shmem.on_rank(part, rank), shmem.on_rank(out, rank),
+                                               shmem.on_rank(flags_dn, rank), hb, rank, ws, grid_dn, bm, bn, 64, 6,
+                                               ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks),
+                    "reduce": "reduce"}
             for name, fn in (("gate_up", up), ("down", down), ("reduce", reduce)):
                 ms = graph_ms(fn, 10, 10)
                 if name not in best or ms < best[name][0]:
-                    best[name] = (ms, [bm, bn], sk[name])
+                    best[name] = (ms, [bm, bn], sk[name], kern[name])
             shmem.heap_offset = hoff
         ms_up, ms_dn, ms_red = best["gate_up"][0], best["down"][0], best["reduce"][0]
         fl = 2.0 * Mt * hidden * ffn
@@ -343,6 +350,7 @@ def run_decoder(args):
         rows.append({
             "M": Mt, "tile_up": best["gate_up"][1], "tile_down": best["down"][1], "tile_reduce": best["reduce"][1],
             "split_k_up": best["gate_up"][2], "split_k_down": best["down"][2],
+            "kernel_up": best["gate_up"][3], "kernel_down": best["down"][3],
             "gate_up_us": round(ms_up * 1e3, 2), "gate_up_tflops": round(fl / ms_up / 1e9, 2),
             "gate_up_weight_GBps": round(wbytes / ms_up / 1e6, 1),
             "down_us": round(ms_dn * 1e3, 2), "down_tflops": round(fl / ms_dn / 1e9, 2),

@@ -99,6 +99,15 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 #define IRIS_STATUS_OK 0
 #define IRIS_STATUS_SPIN_TIMEOUT 1 /* a flag wait gave up; that tile was not reduced */
 
+/* Special values of iris_gemm_args.variant.  A launch with at most 16 rows of
+ * A whose operands are K-contiguous normally takes a kernel of its own that
+ * streams B once (one workgroup per 16 columns of C, no LDS staging);
+ * FEW_ROWS insists on it (hipErrorInvalidValue when the launch does not
+ * qualify), PERSISTENT keeps the default choice among the persistent kernels.
+ * The reference has one Triton kernel for every M (gemm_all_scatter.py:95). */
+#define IRIS_GEMM_VARIANT_FEW_ROWS 1000
+#define IRIS_GEMM_VARIANT_PERSISTENT 1001
+
 /*
  * Arguments of one persistent shard-GEMM launch.  It is the argument list of
  * the reference kernels (gemm_*:95-132) plus what their Triton launch passes
@@ -131,7 +140,7 @@ typedef struct iris_gemm_args {
   int32_t phase;        /* IRIS_PHASE_* (ONE_SHOT only)                           */
   int32_t notify;       /* ALL_SCATTER: publish a ready flag per tile   gemm_*:128 (NOTIFY_REMOTES) */
   int32_t scope;        /* IRIS_SCOPE_*                                           */
-  int32_t variant;      /* 0 = default kernel choice; >0 selects a tuning variant */
+  int32_t variant;      /* 0 = default kernel choice; >0 selects a tuning variant, or IRIS_GEMM_VARIANT_* */
   uint64_t spin_timeout_ticks; /* bound on a flag wait in 100 MHz ticks; 0 = default (2 s) */
   /* Split-K workspace: the `P` and `locks` buffers that matmul.apply receives
    * (matmul_wrapper.py:29-31,73-92; allocated at benchmark.py:136-142).  With both
@@ -161,6 +170,10 @@ int iris_gemm_launch(const iris_gemm_args* args, void* stream);
 int iris_gemm_kernel_info(const iris_gemm_args* args, int* n_regs, int* n_spills);
 /* The split-K factor `iris_gemm_launch` would use for `args` (1 = unsplit). */
 int iris_gemm_split_k(const iris_gemm_args* args, int* split_k);
+
+/* Name of the kernel `iris_gemm_launch` would run for `args` ("" when there is
+ * no GEMM work): a tuning variant's name, or "few_rows_16xN". */
+int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t len);
 
 /* Name of tuning variant `variant` (1-based) of the kernel list used for
  * (ab_dtype, fp32 output?, atomic?); hipErrorInvalidValue past the end. */

@@ -23,6 +23,8 @@ EPI_ALL_SCATTER, EPI_ATOMIC_ADD, EPI_ONE_SHOT = 0, 1, 2
 PHASE_PRODUCE, PHASE_CONSUME, PHASE_FUSED = 1, 2, 3
 # flag scopes (IRIS_SCOPE_*)
 SCOPE_AGENT, SCOPE_SYSTEM = 0, 1
+# special values of GemmArgs.variant (include/iris_amd.h)
+VARIANT_FEW_ROWS, VARIANT_PERSISTENT = 1000, 1001
 # status word (IRIS_STATUS_*)
 STATUS_OK, STATUS_SPIN_TIMEOUT = 0, 1
 
@@ -131,6 +133,7 @@ SIGNATURES = {
     "iris_gemm_kernel_info": (_I, [ctypes.POINTER(GemmArgs), ctypes.POINTER(_I), ctypes.POINTER(_I)]),
     "iris_gemm_split_k": (_I, [ctypes.POINTER(GemmArgs), ctypes.POINTER(_I)]),
     "iris_gemm_variant_name": (_I, [_I, _I, _I, _I, ctypes.c_char_p, ctypes.c_size_t]),
+    "iris_gemm_plan_name": (_I, [ctypes.POINTER(GemmArgs), ctypes.c_char_p, ctypes.c_size_t]),
     "iris_one_shot_reduce_launch": (_I, [ctypes.POINTER(ReduceArgs), _P]),
     "iris_signal_tiles_launch": (_I, [_P, _P, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
                                       ctypes.c_int32, _P]),

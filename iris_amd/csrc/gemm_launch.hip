@@ -3,7 +3,7 @@
 #include <cstdlib>
 #include <mutex>
 
-#include "gemm_registry.hpp"
+#include "gemm_skinny.hpp"
 
 namespace iris_amd {
 
@@ -40,6 +40,9 @@ struct Plan {
   const GemmKernelEntry* entry = nullptr;
   GemmKArgs k{};
   int fused_reduce = 0;  // ONE_SHOT with the CONSUME phase: follow with the reduce kernel
+  // the few-rows kernel instead of a table entry, one workgroup per 16 columns
+  GemmKernelFn skinny = nullptr;
+  int skinny_grid = 0;
 };
 
 int dbg() {
@@ -149,13 +152,40 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
     return ((int64_t)e.cm * a.stride_am + a.K) * 2 < lim && ((int64_t)e.cn * a.stride_bn + a.K) * 2 < lim;
   };
 
+  // At most 16 rows: the product is a stream over B, and the kernel built for
+  // that takes it when the operands allow the 16-byte fetches, the logical
+  // tile covers every row, and the tiles' arrival counters have a home.
+  if (a.variant == 0 || a.variant == IRIS_GEMM_VARIANT_FEW_ROWS) {
+    const int64_t lim = (int64_t)1 << 31;
+    const bool counters = a.block_n <= SKINNY_COLS || a.N <= SKINNY_COLS || k.flag_mode == 0 ||
+                          (a.locks && k.total_tiles <= a.num_sms);
+    const bool ok = a.M <= SKINNY_ROWS && a.K > 0 && dma_ok && (op == OP_STORE16 || op == OP_STORE32) &&
+                    a.block_m >= a.M && (a.block_n % SKINNY_COLS) == 0 && !a.mm_begin_timestamp &&
+                    !a.mm_end_timestamp && a.split_k <= 1 && counters &&
+                    ((int64_t)SKINNY_ROWS * a.stride_am + a.K) * 2 < lim &&
+                    ((int64_t)SKINNY_COLS * a.stride_bn + a.K) * 2 < lim;
+    if (ok) {
+      // fetches in flight per wave: enough for the whole K range, 8 blocks at most
+      const int per_wave = ((a.K + 63) / 64 + SKINNY_WAVES - 1) / SKINNY_WAVES;
+      plan->skinny = gemm_skinny_kernel_for(a.ab_dtype, op, per_wave <= 2 ? 2 : per_wave <= 4 ? 4 : 8);
+      plan->skinny_grid = (a.N + SKINNY_COLS - 1) / SKINNY_COLS;
+      k.split_k = 1;
+      k.locks = a.locks;
+      if (plan->skinny) return hipSuccess;
+    }
+    if (a.variant == IRIS_GEMM_VARIANT_FEW_ROWS) return hipErrorInvalidValue;
+  }
+
   const GemmKernelEntry* pick = nullptr;
-  if (a.variant > 0) {
+  if (a.variant == IRIS_GEMM_VARIANT_PERSISTENT) {
+    // the default choice among the persistent kernels
+  } else if (a.variant > 0) {
     if (a.variant > count) return hipErrorInvalidValue;
     const GemmKernelEntry& e = list[a.variant - 1];
     if (!fits(e)) return hipErrorInvalidValue;
     pick = &e;
-  } else {
+  }
+  if (!pick) {
     // first entry whose compute tile divides the logical tile; the rows and
     // columns a small matrix cannot fill are not worth a tall compute tile
     for (int i = 0; i < count && !pick; ++i) {
@@ -269,7 +299,14 @@ extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
   hipError_t err = make_plan(*args, &plan);
   if (err != hipSuccess) return err;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (plan.entry) {
+  if (plan.skinny) {
+    if (dbg())
+      std::fprintf(stderr, "[iris_amd] gemm few-rows M=%d N=%d K=%d tiles=%d grid=%d\n", plan.k.M, plan.k.N, plan.k.K,
+                   plan.k.total_tiles, plan.skinny_grid);
+    hipLaunchKernelGGL(plan.skinny, dim3(plan.skinny_grid), dim3(SKINNY_THREADS), 0, s, plan.k);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+  } else if (plan.entry) {
     const GemmKernelEntry* e = plan.entry;
     const GemmKernelFn fn = plan.k.split_k > 1 ? e->fn_split : e->fn;
     if (e->lds_bytes > 64 * 1024) {
@@ -299,7 +336,7 @@ extern "C" int iris_gemm_split_k(const iris_gemm_args* args, int* split_k) {
   Plan plan;
   hipError_t err = make_plan(*args, &plan);
   if (err != hipSuccess) return err;
-  *split_k = plan.entry ? plan.k.split_k : 1;
+  *split_k = plan.entry && !plan.skinny ? plan.k.split_k : 1;
   return hipSuccess;
 }
 
@@ -310,9 +347,9 @@ extern "C" int iris_gemm_kernel_info(const iris_gemm_args* args, int* n_regs, in
   if (err != hipSuccess) return err;
   if (n_regs) *n_regs = 0;
   if (n_spills) *n_spills = 0;
-  if (!plan.entry) return hipSuccess;
+  if (!plan.entry && !plan.skinny) return hipSuccess;
   hipFuncAttributes attr;
-  err = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(plan.entry->fn));
+  err = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(plan.skinny ? plan.skinny : plan.entry->fn));
   if (err != hipSuccess) return err;
   if (n_regs) *n_regs = attr.numRegs;
   if (n_spills) *n_spills = static_cast<int>(attr.localSizeBytes);
@@ -325,5 +362,14 @@ extern "C" int iris_gemm_variant_name(int ab_dtype, int out_is_f32, int atomic, 
   const GemmKernelEntry* list = entries_for(ab_dtype, op, &count);
   if (!list || variant < 1 || variant > count || !buf || len == 0) return hipErrorInvalidValue;
   std::snprintf(buf, len, "%s", list[variant - 1].name);
+  return hipSuccess;
+}
+
+extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t len) {
+  if (!args || !buf || len == 0) return hipErrorInvalidValue;
+  Plan plan;
+  hipError_t err = make_plan(*args, &plan);
+  if (err != hipSuccess) return err;
+  std::snprintf(buf, len, "%s", plan.skinny ? "few_rows_16xN" : plan.entry ? plan.entry->name : "");
   return hipSuccess;
 }

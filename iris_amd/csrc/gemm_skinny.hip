@@ -1,0 +1,32 @@
+// Instantiations of the few-rows shard GEMM.
+#include "gemm_skinny.hpp"
+
+namespace iris_amd {
+
+namespace {
+
+template <int DT, int OP>
+GemmKernelFn pick_un(int un) {
+  constexpr int ODT = OP == OP_STORE32 ? IRIS_DTYPE_F32 : DT;
+  switch (un) {
+    case 2: return &gemm_skinny_kernel<DT, OP, ODT, 2>;
+    case 4: return &gemm_skinny_kernel<DT, OP, ODT, 4>;
+    case 8: return &gemm_skinny_kernel<DT, OP, ODT, 8>;
+  }
+  return nullptr;
+}
+
+}  // namespace
+
+GemmKernelFn gemm_skinny_kernel_for(int dt, int op, int un) {
+  if (dt == IRIS_DTYPE_BF16) {
+    if (op == OP_STORE16) return pick_un<IRIS_DTYPE_BF16, OP_STORE16>(un);
+    if (op == OP_STORE32) return pick_un<IRIS_DTYPE_BF16, OP_STORE32>(un);
+  } else if (dt == IRIS_DTYPE_F16) {
+    if (op == OP_STORE16) return pick_un<IRIS_DTYPE_F16, OP_STORE16>(un);
+    if (op == OP_STORE32) return pick_un<IRIS_DTYPE_F16, OP_STORE32>(un);
+  }
+  return nullptr;
+}
+
+}  // namespace iris_amd

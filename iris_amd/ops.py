@@ -25,12 +25,15 @@ from ._native import (
     PHASE_PRODUCE,
     SCOPE_AGENT,
     SCOPE_SYSTEM,
+    VARIANT_FEW_ROWS,
+    VARIANT_PERSISTENT,
 )
 
 __all__ = [
     "gemm_launch",
     "gemm_kernel_info",
     "gemm_split_k",
+    "gemm_plan_name",
     "gemm_variant_name",
     "one_shot_reduce",
     "signal_tiles",
@@ -191,19 +194,24 @@ def _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_s
     args.scope = scope
     args.variant = variant
     args.spin_timeout_ticks = spin_timeout_ticks
-    # split-K workspace: the wrappers' P [num_sms, BLK_M*BLK_N] fp32 and locks [num_sms] int32
-    if (partials is None) != (locks is None):
-        raise ValueError("partials and locks go together")
-    if partials is not None:
-        _require_cuda("partials", partials, device)
+    # workspace: the wrappers' P [num_sms, BLK_M*BLK_N] fp32 and locks [num_sms] int32.  Split-K needs both;
+    # the few-rows kernel only counts arrivals in locks.
+    if partials is not None and locks is None:
+        raise ValueError("partials need locks")
+    if locks is not None:
         _require_cuda("locks", locks, device)
-        if partials.dtype != torch.float32 or partials.dim() != 2 or not partials.is_contiguous():
-            raise TypeError("partials must be a contiguous fp32 matrix [num_sms, BLK_M * BLK_N]")
         if locks.dtype != torch.int32 or not locks.is_contiguous():
             raise TypeError("locks must be a contiguous int32 tensor")
-        if partials.shape[0] < num_sms or locks.numel() < num_sms:
-            raise ValueError("partials and locks need one slot per program")
-        args.partials, args.locks = _ptr(partials), _ptr(locks)
+        if locks.numel() < num_sms:
+            raise ValueError("locks need one slot per program")
+        args.locks = _ptr(locks)
+    if partials is not None:
+        _require_cuda("partials", partials, device)
+        if partials.dtype != torch.float32 or partials.dim() != 2 or not partials.is_contiguous():
+            raise TypeError("partials must be a contiguous fp32 matrix [num_sms, BLK_M * BLK_N]")
+        if partials.shape[0] < num_sms:
+            raise ValueError("partials need one slot per program")
+        args.partials = _ptr(partials)
         args.partials_slot_elems = partials.shape[1]
     elif split_k > 1:
         raise ValueError("split_k > 1 needs the partials and locks workspace")
@@ -251,6 +259,22 @@ def gemm_split_k(a, b, c, c_global, tile_completed, heap_bases, rank, world_size
         raise ValueError("iris_gemm_split_k rejected the arguments")
     _native.hip_try(err)
     return sk.value
+
+
+def gemm_plan_name(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
+                   gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, variant=0, partials=None,
+                   locks=None, split_k=0):
+    """Name of the kernel a launch with these arguments would run."""
+    args = _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N,
+                           BLK_K, gsize_m, epilogue, phase, notify, num_xcds, SCOPE_AGENT, variant, None, None, None,
+                           0, partials, locks, split_k)
+    buf = ctypes.create_string_buffer(128)
+    with torch.cuda.device(a.device):
+        err = _native.lib().iris_gemm_plan_name(ctypes.byref(args), buf, 128)
+    if err == _native.HIP_ERROR_INVALID_VALUE:
+        raise ValueError("iris_gemm_plan_name rejected the arguments")
+    _native.hip_try(err)
+    return buf.value.decode()
 
 
 def gemm_kernel_info(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,

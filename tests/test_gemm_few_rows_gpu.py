@@ -1,0 +1,197 @@
+"""Parity of the few-rows shard GEMM (at most 16 rows of A, one workgroup per
+16 columns of C) against the CPU oracle, through the C-ABI.
+
+Same bar as the persistent kernel: values rtol 1e-2 / atol 1e-2 against the
+fp32-accumulated oracle, flags and arrival counters bit-exact.
+"""
+
+import pytest
+import torch
+
+from iris_amd import ops
+from oracle import iris_oracle as O
+from test_gemm_gpu import check_close, make_ab, to_heap
+
+pytestmark = pytest.mark.gpu
+
+FEW = "few_rows_16xN"
+
+
+def scatter(shmem, a, b, cg, flags, rank, ws, BM, BN, G, *, locks=None, variant=0, notify=True, grid=256):
+    args = (a, b, None, cg, flags, shmem.get_heap_bases(), rank, ws, grid, BM, BN, 64, G, ops.EPI_ALL_SCATTER)
+    name = ops.gemm_plan_name(*args, notify=notify, locks=locks, partials=None, variant=variant)
+    ops.gemm_launch(*args, notify=notify, locks=locks, variant=variant)
+    return name
+
+
+CASES = [
+    # M, N, K, BLK_M, BLK_N, G, dtype
+    (1, 1376, 4096, 256, 256, 4, torch.bfloat16),   # decoder gate/up, one token
+    (16, 1376, 4096, 64, 64, 4, torch.bfloat16),
+    (16, 4096, 1376, 128, 128, 6, torch.bfloat16),  # decoder down: 21 K blocks and a tail of 32
+    (3, 40, 72, 16, 16, 1, torch.bfloat16),         # one workgroup per logical tile; ragged last block; K tail of 8
+    (7, 50, 8, 64, 32, 2, torch.float16),           # N not a multiple of 4: element-wise stores; a single 8-k chunk
+    (16, 16, 64, 16, 16, 1, torch.float16),
+    (5, 272, 9000, 32, 48, 3, torch.bfloat16),      # K range that takes a wave two rounds of fetches
+    (12, 2048, 640, 256, 128, 4, torch.float16),
+]
+
+
+@pytest.mark.parametrize("M,N,K,BM,BN,G,dtype", CASES)
+def test_scatter_single_rank(shmem, M, N, K, BM, BN, G, dtype):
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.full((M, N), 7, dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total + 3,), dtype=torch.int32)
+    locks = shmem.zeros((256,), dtype=torch.int32)
+    for launch in (1, 2):
+        cg.fill_(7)
+        assert scatter(shmem, a, b, cg, flags, 0, 1, BM, BN, G, locks=locks) == FEW
+        torch.cuda.synchronize()
+        check_close(cg, O.shard_gemm(A, B, dtype), f"launch {launch}")
+        # one arrival per tile and launch; the arrival counters are back at zero
+        assert flags.cpu().tolist() == [launch] * total + [0, 0, 0]
+        assert not locks.any()
+
+
+def test_strided_operands_and_output(shmem):
+    """K-shard views (leading dimensions > K) and an output that is a column
+    block of a wider matrix."""
+    M, N, K, dtype = 9, 96, 320, torch.bfloat16
+    A, B = make_ab(M, N, K, dtype, lda=1024, ldb=2048)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    wide = shmem.full((M, 3 * N), 5, dtype=dtype)
+    cg = wide[:, N:2 * N]
+    flags = shmem.zeros((2,), dtype=torch.int32)
+    locks = shmem.zeros((256,), dtype=torch.int32)
+    assert scatter(shmem, a, b, cg, flags, 0, 1, 64, 64, 4, locks=locks) == FEW
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, dtype))
+    assert (wide[:, :N] == 5).all() and (wide[:, 2 * N:] == 5).all()
+    assert flags.cpu().tolist() == [1, 1]
+
+
+@pytest.mark.parametrize("ws", [2, 8])
+def test_scatter_virtual_ranks(shmem, ws):
+    """Rank r's [M, N/ws] block lands at column r*N/ws of c_global on every
+    rank (wave w of a workgroup stores on rank w); every rank's flags count ws
+    arrivals."""
+    M, K, BM, BN, G, dtype = 16, 512, 64, 64, 4, torch.bfloat16
+    N = 176 * ws
+    A, B = make_ab(M, N, K, dtype)
+    shards = O.n_shards(A, B, ws)
+    a = to_heap(shmem, A)
+    bs = [to_heap(shmem, sb) for _, sb in shards]
+    cg = shmem.zeros((M, N), dtype=dtype)
+    n_local = N // ws
+    total = ops.cdiv(n_local, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    locks = shmem.zeros((256,), dtype=torch.int32)
+    for r in range(ws):
+        shmem.on_rank(cg, r).zero_()
+        shmem.on_rank(flags, r).zero_()
+    for r in range(ws):
+        assert scatter(shmem, a, bs[r], shmem.on_rank(cg, r), shmem.on_rank(flags, r), r, ws, BM, BN, G,
+                       locks=shmem.on_rank(locks, r)) == FEW
+    torch.cuda.synchronize()
+    want = O.all_scatter(shards, dtype)
+    for r in range(ws):
+        check_close(shmem.on_rank(cg, r), want, f"rank {r}")
+        assert shmem.on_rank(flags, r).cpu().tolist() == [ws] * total
+        assert not shmem.on_rank(locks, r).any()
+
+
+@pytest.mark.parametrize("pdtype", [torch.float32, torch.bfloat16])
+def test_one_shot_producer_and_reduce(shmem, pdtype):
+    """K-split over 4 ranks: each rank's partial through the few-rows kernel,
+    +1 on every other rank's flag per tile, then the reduce kernel."""
+    ws, M, N, K, BM, BN, G, dtype = 4, 16, 384, 4 * 256, 32, 128, 6, torch.bfloat16
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    shards = O.k_shards(A, B, ws)
+    ah, bh = to_heap(shmem, A), to_heap(shmem, B)
+    kk = K // ws
+    part = shmem.zeros((M, N), dtype=pdtype)
+    out = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(N, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    locks = shmem.zeros((256,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+    for r in range(ws):
+        for t in (part, out, flags, locks):
+            shmem.on_rank(t, r).zero_()
+    for r in range(ws):
+        args = (ah[:, r * kk:(r + 1) * kk], bh[r * kk:(r + 1) * kk, :], shmem.on_rank(part, r), shmem.on_rank(out, r),
+                shmem.on_rank(flags, r), hb, r, ws, 256, BM, BN, 64, G, ops.EPI_ONE_SHOT)
+        kw = dict(phase=ops.PHASE_PRODUCE, locks=shmem.on_rank(locks, r))
+        assert ops.gemm_plan_name(*args, **kw) == FEW
+        ops.gemm_launch(*args, **kw)
+    torch.cuda.synchronize()
+    for r in range(ws):
+        check_close(shmem.on_rank(part, r), O.shard_gemm(*shards[r], pdtype), f"partial {r}")
+        assert shmem.on_rank(flags, r).cpu().tolist() == [ws - 1] * total  # every other rank arrived once
+    for r in range(ws):
+        ops.one_shot_reduce(shmem.on_rank(part, r), shmem.on_rank(out, r), shmem.on_rank(flags, r), hb, r, ws, BM,
+                            BN, G)
+    torch.cuda.synchronize()
+    want = O.one_shot_all_reduce(shards, pdtype, dtype)
+    for r in range(ws):
+        check_close(shmem.on_rank(out, r), want, f"reduced on rank {r}")
+        assert not shmem.on_rank(flags, r).any()
+
+
+def test_choice_of_kernel(shmem):
+    dtype = torch.bfloat16
+    A, B = make_ab(16, 256, 128, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((16, 256), dtype=dtype)
+    flags = shmem.zeros((64,), dtype=torch.int32)
+    locks = shmem.zeros((256,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+
+    def plan(a_, b_, cg_, BM, BN, **kw):
+        return ops.gemm_plan_name(a_, b_, None, cg_, flags, hb, 0, 1, 256, BM, BN, 64, 4, ops.EPI_ALL_SCATTER, **kw)
+
+    assert plan(a, b, cg, 64, 64, locks=locks) == FEW
+    assert plan(a, b, cg, 64, 64, locks=locks, variant=ops.VARIANT_FEW_ROWS) == FEW
+    # several workgroups per flag and nowhere to count their arrivals
+    assert plan(a, b, cg, 64, 64) != FEW
+    # ... unless nothing is published, or a flag belongs to one workgroup
+    assert plan(a, b, cg, 64, 64, notify=False) == FEW
+    assert plan(a, b, cg, 16, 16) == FEW
+    # the persistent kernels on request
+    assert plan(a, b, cg, 64, 64, locks=locks, variant=ops.VARIANT_PERSISTENT) == "64x64x64_w2x2_s4"
+    assert plan(a, b, cg, 64, 64, locks=locks, variant=6) == "64x64x64_w2x2_s4"
+    # a logical tile that does not cover the rows, or is no multiple of 16 columns
+    assert plan(a, b, cg, 8, 64, locks=locks) != FEW
+    assert plan(a, b, cg, 64, 40, locks=locks) != FEW
+    # more than 16 rows
+    A2, B2 = make_ab(17, 256, 128, dtype)
+    a2, cg2 = to_heap(shmem, A2), shmem.zeros((17, 256), dtype=dtype)
+    assert plan(a2, b, cg2, 64, 64, locks=locks) != FEW
+    with pytest.raises(ValueError):
+        plan(a2, b, cg2, 64, 64, locks=locks, variant=ops.VARIANT_FEW_ROWS)
+    # B with N contiguous: no 16-byte fetches along K
+    bn = shmem.zeros((128, 256), dtype=dtype)
+    assert plan(a, bn, cg, 64, 64, locks=locks) != FEW
+    # atomics keep the persistent kernel
+    assert ops.gemm_plan_name(a, b, None, cg, flags, hb, 0, 1, 256, 64, 64, 64, 4, ops.EPI_ATOMIC_ADD,
+                              locks=locks) != FEW
+
+
+def test_persistent_choice_gives_the_same_result(shmem):
+    """The two kernels on one input: same values to the parity tolerance, same flags."""
+    M, N, K, dtype = 16, 1376, 1024, torch.bfloat16
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    locks = shmem.zeros((256,), dtype=torch.int32)
+    got = {}
+    for variant in (0, ops.VARIANT_PERSISTENT):
+        cg = shmem.zeros((M, N), dtype=dtype)
+        flags = shmem.zeros((ops.cdiv(N, 128),), dtype=torch.int32)
+        name = scatter(shmem, a, b, cg, flags, 0, 1, 128, 128, 4, locks=locks, variant=variant)
+        torch.cuda.synchronize()
+        got[variant] = (name, cg, flags.cpu().tolist())
+    assert got[0][0] == FEW and got[ops.VARIANT_PERSISTENT][0] != FEW
+    check_close(got[0][1], got[ops.VARIANT_PERSISTENT][1])
+    assert got[0][2] == got[ops.VARIANT_PERSISTENT][2]
