@@ -437,9 +437,9 @@ def test_split_k_all_scatter(shmem, M, N, K, BM, BN, split_k, dtype):
 
 def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
     dtype = torch.bfloat16
-    A, B = make_ab(16, 1376, 4096, dtype)
+    A, B = make_ab(40, 1376, 4096, dtype)  # (up to 16 rows would go to the few-rows kernel)
     a, b = to_heap(shmem, A), to_heap(shmem, B)
-    cg = shmem.zeros((16, 1376), dtype=dtype)
+    cg = shmem.zeros((40, 1376), dtype=dtype)
     flags = shmem.zeros((32,), dtype=torch.int32)
     partials, locks = split_workspace(shmem, 256, 64, 64)
     common = (a, b, None, cg, flags, None, 0, 1, 256, 64, 64, 64, 4, ops.EPI_ALL_SCATTER)
