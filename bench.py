@@ -300,18 +300,20 @@ def run_decoder(args):
             flags_up = shmem.zeros((t_up,), dtype=torch.int32)
             flags_dn = shmem.zeros((t_dn,), dtype=torch.int32)
             grid_up = grid_dn = 256
+            xcds = ops.default_num_xcds(shmem.get_cu_count(), 256)  # what the matmul wrappers pass
             # the wrappers' P / locks buffers: with them the launcher may split K over idle programs
             P = shmem.zeros((256, bm * bn), dtype=torch.float32)
             locks = shmem.zeros((256,), dtype=torch.int32)
 
             def up():
                 ops.gemm_launch(x, wg.T, None, shmem.on_rank(gate_all, rank), shmem.on_rank(flags_up, rank), hb, rank,
-                                ws, grid_up, bm, bn, 64, 4, ops.EPI_ALL_SCATTER, notify=True, partials=P, locks=locks)
+                                ws, grid_up, bm, bn, 64, 4, ops.EPI_ALL_SCATTER, notify=True, partials=P, locks=locks,
+                                num_xcds=xcds)
 
             def down():
                 ops.gemm_launch(h, wd.T, shmem.on_rank(part, rank), shmem.on_rank(out, rank),
                                 shmem.on_rank(flags_dn, rank), hb, rank, ws, grid_dn, bm, bn, 64, 6,
-                                ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks)
+                                ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks, num_xcds=xcds)
 
             def reduce():
                 ops.one_shot_reduce(shmem.on_rank(part, rank), shmem.on_rank(out, rank),

@@ -53,6 +53,10 @@ struct GemmKArgs {
   int M, N, K;
   int BM, BN, G;
   int num_sms, num_xcds, cur_rank, ws;
+  // > 0: fewer work items than programs.  The reference remap would leave
+  // whole XCDs idle then; instead each XCD takes xcd_per consecutive items
+  // (neighbouring tiles, whose operand panels its L2 then fetches once).
+  int xcd_per;
   int num_pid_m, num_pid_n, total_tiles;
   int sub_m, sub_n;  // compute tiles per logical tile
   int dest_all;      // write `out` on every rank's heap (else on this rank only)
@@ -646,7 +650,14 @@ gemm_persistent_kernel(const GemmKArgs p) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
-  const int pid = xcd_remap(blockIdx.x, p.num_sms, p.num_xcds);
+  int pid;
+  if (p.xcd_per > 0) {
+    // workgroups are dealt to the XCDs round-robin: this one is number j on XCD x
+    const int x = blockIdx.x % p.num_xcds, j = blockIdx.x / p.num_xcds;
+    pid = j < p.xcd_per ? x * p.xcd_per + j : p.num_sms * 2;  // (past every item: nothing to do)
+  } else {
+    pid = xcd_remap(blockIdx.x, p.num_sms, p.num_xcds);
+  }
 
   constexpr bool split = SPLIT;
   const int work = split ? p.total_tiles * p.split_k : p.total_tiles;  // tiles, or (tile, part) pairs

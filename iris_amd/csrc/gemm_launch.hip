@@ -248,6 +248,10 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
     k.split_q = nk / k.split_k;
     k.split_r = nk % k.split_k;
   }
+  // Fewer (tile, part) items than programs: deal them to the XCDs evenly, in
+  // consecutive runs, instead of filling the first XCDs and idling the rest.
+  const int64_t work = (int64_t)k.total_tiles * k.split_k;
+  if (a.num_xcds > 1 && work < a.num_sms) k.xcd_per = (int)((work + a.num_xcds - 1) / a.num_xcds);
   return hipSuccess;
 }
 
