@@ -9,10 +9,12 @@ positional signature of the reference's three (identical) wrappers
 place of the Triton one (:109-150).
 
 Arguments that only steer the Triton compiler (``num_stages``, ``num_warps``,
-``waves_per_eu``, ``mfmaInstrSize``, ``kpack``) and the dead stream-K buffers
-(``P``, ``locks``, ``two_tiles``) are accepted and ignored; ``BLK_K`` does not
-change any result.  ``bias`` is never applied (the reference forces
-``BIAS=False``, matmul_wrapper.py:104).
+``waves_per_eu``, ``mfmaInstrSize``, ``kpack``) and ``two_tiles`` are accepted
+and ignored; ``BLK_K`` does not change any result.  ``P`` and ``locks``, which
+the reference allocates and never reads, serve as workspace when they have
+the reference's shapes (split-K partials; arrival counters of the few-rows
+kernel) and are ignored otherwise.  ``bias`` is never applied (the reference
+forces ``BIAS=False``, matmul_wrapper.py:104).
 """
 
 from __future__ import annotations
