@@ -42,7 +42,7 @@ struct Plan {
   int fused_reduce = 0;  // ONE_SHOT with the CONSUME phase: follow with the reduce kernel
   // the few-rows kernel instead of a table entry, one workgroup per 16 columns
   GemmKernelFn skinny = nullptr;
-  int skinny_grid = 0;
+  int skinny_grid = 0, skinny_lds = 0;
 };
 
 int dbg() {
@@ -167,7 +167,9 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
     if (ok) {
       // fetches in flight per wave: enough for the whole K range, 8 blocks at most
       const int per_wave = ((a.K + 63) / 64 + SKINNY_WAVES - 1) / SKINNY_WAVES;
-      plan->skinny = gemm_skinny_kernel_for(a.ab_dtype, op, per_wave <= 2 ? 2 : per_wave <= 4 ? 4 : 8);
+      const int un = per_wave <= 2 ? 2 : per_wave <= 4 ? 4 : 8;
+      plan->skinny = gemm_skinny_kernel_for(a.ab_dtype, op, un);
+      plan->skinny_lds = skinny_lds_bytes(un);
       plan->skinny_grid = (a.N + SKINNY_COLS - 1) / SKINNY_COLS;
       k.split_k = 1;
       k.locks = a.locks;
@@ -255,12 +257,12 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   return hipSuccess;
 }
 
-hipError_t ensure_lds(const GemmKernelEntry* e, GemmKernelFn fn) {
+hipError_t ensure_lds(GemmKernelFn fn, int lds_bytes) {
   // dynamic LDS above 64 KiB must be opted into once per function
   static std::mutex m;
   std::lock_guard<std::mutex> lock(m);
   return hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                             e->lds_bytes);
+                             lds_bytes);
 }
 
 iris_reduce_args reduce_args_from(const iris_gemm_args& a) {
@@ -307,14 +309,18 @@ extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
     if (dbg())
       std::fprintf(stderr, "[iris_amd] gemm few-rows M=%d N=%d K=%d tiles=%d grid=%d\n", plan.k.M, plan.k.N, plan.k.K,
                    plan.k.total_tiles, plan.skinny_grid);
-    hipLaunchKernelGGL(plan.skinny, dim3(plan.skinny_grid), dim3(SKINNY_THREADS), 0, s, plan.k);
+    if (plan.skinny_lds > 64 * 1024) {
+      err = ensure_lds(plan.skinny, plan.skinny_lds);
+      if (err != hipSuccess) return err;
+    }
+    hipLaunchKernelGGL(plan.skinny, dim3(plan.skinny_grid), dim3(SKINNY_THREADS), plan.skinny_lds, s, plan.k);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
   } else if (plan.entry) {
     const GemmKernelEntry* e = plan.entry;
     const GemmKernelFn fn = plan.k.split_k > 1 ? e->fn_split : e->fn;
     if (e->lds_bytes > 64 * 1024) {
-      err = ensure_lds(e, fn);
+      err = ensure_lds(fn, e->lds_bytes);
       if (err != hipSuccess) return err;
     }
     if (dbg())

@@ -4,12 +4,19 @@
 //
 // With so few rows the product is a stream over B: every byte of B is used
 // once, the matrix cores idle, and what matters is how many bytes a CU has in
-// flight.  So nothing goes through LDS: a workgroup of eight waves owns 16
-// columns of C, its waves share the K range out in blocks of 64, and a lane
-// fetches its MFMA operands straight into registers, 32 contiguous bytes of a
-// row of B (and of A) per block, every fetch of a wave issued before the
-// first MFMA.  The eight partial 16x16 accumulators meet in LDS; wave w then
-// stores the sum on destination rank w, w+8, ...
+// flight and how many bytes each cache-line access of its L1 brings.  A
+// workgroup of eight waves owns 16 columns of C and its waves share the K
+// range out in blocks of 64.  Every fetch of a wave is issued before its
+// first MFMA:
+//   * B, the stream, comes in with `buffer_load ... lds`, one instruction per
+//     8 rows x 128 bytes (whole cache lines: twice the bytes per line access
+//     of a fetch in MFMA operand layout, 16 rows x 64 bytes), into a region of
+//     LDS private to the wave, 16-byte chunks XOR-ed by the row so that the
+//     operand reads are conflict-free;
+//   * A, at most 16 rows that every workgroup reads and L2 holds, goes
+//     straight into registers in operand layout.
+// The eight partial 16x16 accumulators meet in LDS; wave w then stores the
+// sum on destination rank w, w+8, ...
 //
 // A logical tile (BLOCK_SIZE_M x BLOCK_SIZE_N, one flag) spans several such
 // workgroups.  They count their arrivals in locks[tile_id]; the last one to
@@ -24,6 +31,9 @@ constexpr int SKINNY_ROWS = 16;    // rows of A a launch can take
 constexpr int SKINNY_COLS = 16;    // columns of C per workgroup
 constexpr int SKINNY_WAVES = 8;
 constexpr int SKINNY_THREADS = SKINNY_WAVES * 64;
+constexpr int SKINNY_RED_BYTES = SKINNY_WAVES * 64 * 16;  // the waves' partial accumulators
+constexpr int SKINNY_BLOCK_BYTES = 2048;                  // 16 rows of B x 64 k
+constexpr int skinny_lds_bytes(int un) { return SKINNY_RED_BYTES + SKINNY_WAVES * un * SKINNY_BLOCK_BYTES; }
 
 // UN: K blocks (64 k each) whose fetches a wave has in flight together.
 template <int DT, int OP, int ODT, int UN>
@@ -31,13 +41,17 @@ __global__ __launch_bounds__(SKINNY_THREADS) __attribute__((amdgpu_waves_per_eu(
 gemm_skinny_kernel(const GemmKArgs p) {
   static_assert(OP == OP_STORE16 || OP == OP_STORE32, "store epilogues only");
   using vec8 = typename Mfma<DT>::vec8;
-  __shared__ f32x4 red[SKINNY_WAVES][64];
+  extern __shared__ __attribute__((aligned(1024))) char skinny_lds[];
+  IRIS_LDS char* lds = (IRIS_LDS char*)skinny_lds;
+  // [SKINNY_WAVES][64] partial accumulators, then each wave's UN blocks of B
+  IRIS_LDS f32x4* red = (IRIS_LDS f32x4*)lds;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int lr = lane & 15, lq = lane >> 4;
   const int n0 = blockIdx.x * SKINNY_COLS;
+  IRIS_LDS char* wb = lds + SKINNY_RED_BYTES + wave * (UN * SKINNY_BLOCK_BYTES);
 
   // Rows past the edge of either operand lie past the end of its buffer
   // descriptor and read as zero; chunks past K are parked out of range.
@@ -46,50 +60,67 @@ gemm_skinny_kernel(const GemmKArgs p) {
       (void*)(p.b + (int64_t)n0 * p.sbn * 2), 0, (int)((((int64_t)rows_b - 1) * p.sbn + p.K) * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
       (void*)p.a, 0, (int)((((int64_t)p.M - 1) * p.sam + p.K) * 2), 0x00020000);
-  // Lane l holds row l%16 of its operand.  In K block kb, MFMA h (0, 1) takes
-  // k = kb*64 + (l/16)*16 + h*8 .. +7 at MFMA position (l/16)*8 .. +7: the same
-  // permutation of k for both operands, so the products pair up as they
-  // should, and the two fetches of a lane are 32 contiguous bytes.
-  const uint32_t ob = (uint32_t)(((int64_t)lr * p.sbn + lq * 16) * 2);
+  // B: lane l of fetch j of a block brings row 8j + l/8 and lands at byte
+  // l*16 of the fetch's 1 KiB, i.e. at physical chunk l%8 of that row; the
+  // chunk of the row it must bring there is (l%8) ^ (row/2 % 8).
+  const int brow = lane >> 3;  // + 8j
+  const int bchunk = (lane & 7) ^ ((brow >> 1) & 7);  // rows 8j + .. : (row/2)%8 = 4j + brow/2, and 4j flips bit 2
+  // A and the operand reads: lane l holds row l%16.  In K block kb, MFMA h
+  // (0, 1) takes k = kb*64 + (l/16)*16 + h*8 .. +7 at MFMA position
+  // (l/16)*8 .. +7: the same permutation of k for both operands.
   const uint32_t oa = (uint32_t)(((int64_t)lr * p.sam + lq * 16) * 2);
   const int nb = (p.K + 63) / 64;
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int b0 = wave; b0 < nb; b0 += SKINNY_WAVES * UN) {
-    vec8 fb[UN][2], fa[UN][2];
+    vec8 fa[UN][2];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int kb = b0 + SKINNY_WAVES * u;
 #pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int ch = bchunk ^ (j << 2);
+        const bool ok = kb < nb && kb * 64 + ch * 8 < p.K;
+        const uint32_t off = (uint32_t)(((int64_t)(brow + 8 * j) * p.sbn) * 2 + kb * 128 + ch * 16);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (IRIS_LDS void*)(wb + u * SKINNY_BLOCK_BYTES + j * 1024), 16,
+                                                 ok ? (int)off : (int)0x80000000, 0, 0, 0);
+      }
+#pragma unroll
       for (int h = 0; h < 2; ++h) {
         const bool ok = kb < nb && kb * 64 + lq * 16 + h * 8 < p.K;
-        const uint32_t koff = (uint32_t)(kb * 128 + h * 16);
-        fb[u][h] = __builtin_bit_cast(
-            vec8, __builtin_amdgcn_raw_buffer_load_b128(rb, ok ? (int)(ob + koff) : (int)0x80000000, 0, 0));
         fa[u][h] = __builtin_bit_cast(
-            vec8, __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? (int)(oa + koff) : (int)0x80000000, 0, 0));
+            vec8, __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? (int)(oa + kb * 128 + h * 16) : (int)0x80000000, 0, 0));
       }
     }
-    // every fetch is on its way before the first product waits for one
-    __builtin_amdgcn_sched_barrier(0);
+    // every fetch is on its way; B has landed in this wave's own region once
+    // the wave's counter says so (nobody else reads or writes it)
+    IRIS_WAIT_VMCNT(0);
+    asm volatile("" ::: "memory");
 #pragma unroll
     for (int u = 0; u < UN; ++u)
 #pragma unroll
-      for (int h = 0; h < 2; ++h) acc = Mfma<DT>::run(fb[u][h], fa[u][h], acc);
+      for (int h = 0; h < 2; ++h) {
+        const int pc = (lq * 2 + h) ^ ((lr >> 1) & 7);
+        const vec8 fb = *reinterpret_cast<const IRIS_LDS vec8*>(wb + u * SKINNY_BLOCK_BYTES + lr * 128 + pc * 16);
+        acc = Mfma<DT>::run(fb, fa[u][h], acc);
+      }
+    // the reads above have returned before the next round overwrites the region
+    IRIS_WAIT_LGKMCNT0();
+    asm volatile("" ::: "memory");
   }
 
   // acc: row m = l%16 of C, columns n0 + 4*(l/16) .. +3 (operands swapped, as
   // in the persistent kernel)
-  red[wave][lane] = acc;
+  red[wave * 64 + lane] = acc;
   __syncthreads();
 
   const int r_begin = p.dest_all ? 0 : p.cur_rank;
   const int r_end = p.dest_all ? p.ws : p.cur_rank + 1;
   const int m = lr, n = n0 + lq * 4;
   if (r_begin + wave < r_end && m < p.M && n < p.N) {
-    f32x4 s = red[0][lane];
+    f32x4 s = red[lane];
 #pragma unroll
-    for (int w = 1; w < SKINNY_WAVES; ++w) s += red[w][lane];  // wave order: the sum does not depend on timing
+    for (int w = 1; w < SKINNY_WAVES; ++w) s += red[w * 64 + lane];  // wave order: the sum does not depend on timing
     constexpr int ES = OP == OP_STORE32 ? 4 : 2;
     const bool whole = p.vec_out && n + 4 <= p.N;
     for (int r = r_begin + wave; r < r_end; r += SKINNY_WAVES) {
