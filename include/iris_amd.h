@@ -108,6 +108,15 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 #define IRIS_GEMM_VARIANT_FEW_ROWS 1000
 #define IRIS_GEMM_VARIANT_PERSISTENT 1001
 
+/* Special value of iris_gemm_args.split_k: cut the launch's K-steps (all
+ * tiles, in tile order) into num_sms equal runs that start and end anywhere
+ * in a tile, the stream-K schedule the reference's wrappers describe and size
+ * their `P` / `locks` buffers for (matmul_wrapper.py:73-92,
+ * images/stream_k.excalidraw.svg) but do not implement.  Needs partials and
+ * locks; hipErrorInvalidValue when the launch cannot be cut this way.
+ * iris_gemm_split_k reports this value when the launcher chose it itself. */
+#define IRIS_GEMM_SPLIT_STREAM_K (-1)
+
 /*
  * Arguments of one persistent shard-GEMM launch.  It is the argument list of
  * the reference kernels (gemm_*:95-132) plus what their Triton launch passes
@@ -152,7 +161,7 @@ typedef struct iris_gemm_args {
   float* partials;      /* [num_sms][partials_slot_elems] fp32, or NULL           */
   int32_t* locks;       /* int32[num_sms], or NULL                                */
   int64_t partials_slot_elems; /* >= block_m * block_n                            */
-  int32_t split_k;      /* 0 = let the launcher decide, 1 = never, n > 1 = force n */
+  int32_t split_k;      /* 0 = let the launcher decide, 1 = never, n > 1 = force n, IRIS_GEMM_SPLIT_STREAM_K */
   int32_t reserved0;
 } iris_gemm_args;
 

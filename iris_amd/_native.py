@@ -25,6 +25,7 @@ PHASE_PRODUCE, PHASE_CONSUME, PHASE_FUSED = 1, 2, 3
 SCOPE_AGENT, SCOPE_SYSTEM = 0, 1
 # special values of GemmArgs.variant (include/iris_amd.h)
 VARIANT_FEW_ROWS, VARIANT_PERSISTENT = 1000, 1001
+SPLIT_STREAM_K = -1  # GemmArgs.split_k: stream-K
 # status word (IRIS_STATUS_*)
 STATUS_OK, STATUS_SPIN_TIMEOUT = 0, 1
 

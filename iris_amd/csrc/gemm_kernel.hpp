@@ -69,6 +69,13 @@ struct GemmKArgs {
   // `locks[slot]`; the owner adds them in part order and runs the epilogue.
   int split_k;  // >= 1
   int split_q, split_r;  // K-steps per part: nk / split_k and nk % split_k (the first split_r parts take one more)
+  // Stream-K (with split_k == 1): the launch's total_tiles * nk K-steps, in
+  // tile order, are cut into num_sms equal runs, split_q steps each and one
+  // more for the first split_r programs; a run starts and ends anywhere in a
+  // tile.  The program whose run holds a tile's first step owns the tile; the
+  // programs that follow it hold the rest and hand it over through
+  // partials[program] / locks[program] as split-K parts do.
+  int stream_k;
   float* partials;
   int32_t* locks;
   int64_t partial_stride;
@@ -145,17 +152,54 @@ struct Item {
 // Split-K: item `item` of program `pid` is part `part` of tile `slot / split_k`
 // and covers K-steps [k_begin, k_end).  Kept out of Item: these live in
 // scalar registers across the K loop only where they are needed.
+// part 0 owns the tile: its partial-sum slot is `slot`, and the other parts
+// leave theirs in the slots that follow (their own `slot`).
 struct KRange {
   int k_begin, k_end, part, slot;
 };
+// Stream-K: a program's run of global K-steps [g0, g1) starts at step k0 of
+// tile `tile0`.  Computed once per program (it takes a division).
+struct StreamRun {
+  int tile0, k0, g1;
+};
+__device__ inline int stream_len(const GemmKArgs& p, int pid) { return p.split_q + (pid < p.split_r ? 1 : 0); }
+__device__ inline StreamRun stream_run(const GemmKArgs& p, int pid, int nk) {
+  StreamRun r;
+  const int g0 = pid * p.split_q + min(pid, p.split_r);
+  r.g1 = g0 + stream_len(p, pid);
+  r.tile0 = nk > 0 ? g0 / nk : 0;
+  r.k0 = g0 - r.tile0 * nk;
+  return r;
+}
+// Items (tiles touched) of the run.
+__device__ inline int stream_items(const StreamRun& r, int nk) {
+  return r.g1 > r.tile0 * nk + r.k0 ? (r.g1 - 1) / nk - r.tile0 + 1 : 0;
+}
+// Parts of a tile whose owner, program `pid`, stops at step k_end: itself and
+// the programs that hold the rest (each run is at least one step long).
+__device__ inline int stream_parts(const GemmKArgs& p, int pid, int k_end, int nk) {
+  int parts = 1;
+  for (int rem = nk - k_end, q = pid + 1; rem > 0; ++q, ++parts) rem -= stream_len(p, q);
+  return parts;
+}
+// Split-K proper is the same thing with runs that never cross a tile: program
+// pid is part pid % split_k of tile pid / split_k (one item per program).
+__device__ inline StreamRun split_run(const GemmKArgs& p, int pid, int nk) {
+  StreamRun r;
+  r.tile0 = (int)((unsigned)pid / (unsigned)p.split_k);
+  const int part = pid - r.tile0 * p.split_k;
+  r.k0 = part * p.split_q + min(part, p.split_r);
+  r.g1 = r.tile0 * nk + r.k0 + (r.tile0 < p.total_tiles ? p.split_q + (part < p.split_r ? 1 : 0) : 0);
+  return r;
+}
 template <class Cfg, bool SPLIT>
-__device__ inline KRange k_range(const GemmKArgs& p, int pid, int item, int nk) {
+__device__ inline KRange k_range(const GemmKArgs& p, const StreamRun& sr, int pid, int item, int nk) {
   KRange r;
   if constexpr (SPLIT) {
-    r.slot = pid + item * p.num_sms;
-    r.part = (int)((unsigned)r.slot % (unsigned)p.split_k);
-    r.k_begin = r.part * p.split_q + min(r.part, p.split_r);
-    r.k_end = r.k_begin + p.split_q + (r.part < p.split_r ? 1 : 0);
+    r.k_begin = item == 0 ? sr.k0 : 0;
+    r.k_end = min(nk, sr.g1 - (sr.tile0 + item) * nk);
+    r.part = r.k_begin == 0 ? 0 : 1;
+    r.slot = pid;
   } else {
     r.slot = 0;
     r.part = 0;
@@ -166,13 +210,13 @@ __device__ inline KRange k_range(const GemmKArgs& p, int pid, int item, int nk) 
 }
 
 template <class Cfg, bool SPLIT>
-__device__ inline Item decode_item(const GemmKArgs& p, int pid, int item) {
+__device__ inline Item decode_item(const GemmKArgs& p, const StreamRun& sr, int pid, int item) {
   const int subs = p.sub_m * p.sub_n;
   Item it;
   if constexpr (SPLIT) {
-    // one compute tile per logical tile; items are (tile, part) pairs dealt
-    // out to the programs like tiles are
-    it.tile_id = (int)((unsigned)(pid + item * p.num_sms) / (unsigned)p.split_k);
+    // one compute tile per logical tile; the program's run touches tiles
+    // tile0, tile0 + 1, ...
+    it.tile_id = sr.tile0 + item;
     const TileCoord tc = tile_map(it.tile_id, p.num_pid_m, p.num_pid_n, p.G);
     it.lm0 = it.m0 = tc.pid_m * p.BM;
     it.ln0 = it.n0 = tc.pid_n * p.BN;
@@ -613,15 +657,16 @@ __device__ inline void dump_partial(const GemmKArgs& p, const f32x4 (&acc)[Cfg::
                                              ((i * Cfg::IN + j) * Cfg::NT + tid) * 16, 0, 16);
 }
 // acc += partials of parts [q0, q0 + GROUP) of the tile whose part 0 is `slot0`,
-// in part order; parts >= split_k read as zero.  All loads of the group are in
+// in part order; parts >= `parts` read as zero.  All loads of the group are in
 // flight together.
 template <class Cfg, int GROUP>
-__device__ inline void add_partials(const GemmKArgs& p, f32x4 (&acc)[Cfg::IM][Cfg::IN], int slot0, int q0, int tid) {
+__device__ inline void add_partials(const GemmKArgs& p, f32x4 (&acc)[Cfg::IM][Cfg::IN], int slot0, int q0, int parts,
+                                    int tid) {
   constexpr int NB = Cfg::IM * Cfg::IN;
   u32x4 v[GROUP][NB];
 #pragma unroll
   for (int g = 0; g < GROUP; ++g) {
-    const bool present = q0 + g < p.split_k;
+    const bool present = q0 + g < parts;
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(p.partials + (int64_t)(slot0 + (present ? q0 + g : 0)) * p.partial_stride), 0,
         present ? Cfg::CM * Cfg::CN * 4 : 0, 0x00020000);
@@ -660,10 +705,15 @@ gemm_persistent_kernel(const GemmKArgs p) {
   }
 
   constexpr bool split = SPLIT;
+  const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
   const int work = split ? p.total_tiles * p.split_k : p.total_tiles;  // tiles, or (tile, part) pairs
   const int n_mine = pid < work ? (work - pid + p.num_sms - 1) / p.num_sms : 0;
-  const int n_items = split ? n_mine : n_mine * p.sub_m * p.sub_n;
-  const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
+  int n_items = split ? n_mine : n_mine * p.sub_m * p.sub_n;
+  StreamRun sr{0, 0, 0};
+  if constexpr (SPLIT) {
+    sr = p.stream_k ? stream_run(p, pid, nk) : split_run(p, pid, nk);
+    n_items = stream_items(sr, nk);
+  }
   const int total_steps = n_items * nk;  // > 0 iff there is anything to load
 
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
@@ -703,7 +753,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
 
   int c_item = 0;  // compute cursor
   Item c_it;
-  if (n_items > 0) c_it = decode_item<Cfg, SPLIT>(p, pid, 0);
+  if (n_items > 0) c_it = decode_item<Cfg, SPLIT>(p, sr, pid, 0);
 
   // end of a compute tile: store it, and publish the logical tile it completes
   auto epilogue = [&]() __attribute__((always_inline)) {
@@ -715,7 +765,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       pending_tile = -1;
     }
     if constexpr (SPLIT) {
-      const KRange kr = k_range<Cfg, SPLIT>(p, pid, c_item, nk);
+      const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, c_item, nk);
       if (kr.part != 0) {
         // not the owner: leave the partial, raise the lock once every wave's
         // stores have completed, and move on
@@ -723,18 +773,19 @@ gemm_persistent_kernel(const GemmKArgs p) {
         IRIS_WAIT_VMCNT(0);
         __syncthreads();
         if (tid == 0) flag_add_relaxed((IRIS_GLOBAL int32_t*)(p.locks + kr.slot), 1, false);
-        if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, pid, c_item);
+        if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, sr, pid, c_item);
         return;
       }
       // Wait for every other part at once: lane q of the group takes part q's
       // lock (1 -> 0, which also re-arms it for the next launch), each wait
       // bounded; then fetch the partials a few parts at a time.
       int ok = 1;
-      if (tid >= 1 && tid < p.split_k)
+      const int parts = p.stream_k ? stream_parts(p, pid, kr.k_end, nk) : p.split_k;
+      if (tid >= 1 && tid < parts)
         ok = wait_tile_flag((IRIS_GLOBAL int32_t*)(p.locks + kr.slot + tid), 2, false, p.timeout, p.status) ? 1 : 0;
       if (__syncthreads_and(ok)) {
         constexpr int GROUP = Cfg::IM * Cfg::IN * 4 <= 16 ? 4 : Cfg::IM * Cfg::IN * 4 <= 32 ? 2 : 1;
-        for (int q = 1; q < p.split_k; q += GROUP) add_partials<Cfg, GROUP>(p, acc, kr.slot, q, tid);
+        for (int q = 1; q < parts; q += GROUP) add_partials<Cfg, GROUP>(p, acc, kr.slot, q, parts, tid);
       }
     }
     const bool fast = store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN,
@@ -753,7 +804,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
         __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + c_it.tile_id),
                                (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, pid, c_item);
+    if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, sr, pid, c_item);
   };
   auto stamp_begin = [&]() __attribute__((always_inline)) {
     if (p.ts_begin && c_it.first_sub && tid == 0)
@@ -778,8 +829,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
     auto advance_load_cursor = [&]() __attribute__((always_inline)) {
       if (++l_k == l_kend) {
         if (++l_item < n_items) {
-          l_it = decode_item<Cfg, SPLIT>(p, pid, l_item);
-          const KRange kr = k_range<Cfg, SPLIT>(p, pid, l_item, nk);
+          l_it = decode_item<Cfg, SPLIT>(p, sr, pid, l_item);
+          const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, l_item, nk);
           l_k = kr.k_begin;
           l_kend = kr.k_end;
           ld.setup(p, l_it, wave, lane, l_k);
@@ -794,8 +845,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
     };
     Frags<Cfg> fr;
     if (total_steps > 0) {
-      l_it = decode_item<Cfg, SPLIT>(p, pid, 0);
-      const KRange kr = k_range<Cfg, SPLIT>(p, pid, 0, nk);
+      l_it = decode_item<Cfg, SPLIT>(p, sr, pid, 0);
+      const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, 0, nk);
       l_k = kr.k_begin;
       l_kend = kr.k_end;
       ld.setup(p, l_it, wave, lane, l_k);
@@ -912,7 +963,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       stamp_begin();
       run_step(g, std::true_type{});
       ++g;
-      const KRange kr = k_range<Cfg, SPLIT>(p, pid, it, nk);
+      const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, it, nk);
       const int steps = kr.k_end - kr.k_begin;
       for (int k = 1; k < steps; ++k, ++g) run_step(g, std::false_type{});
       epilogue();
@@ -923,7 +974,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
     Frags<Cfg> fr;
     for (int it = 0; it < n_items; ++it) {
       stamp_begin();
-      const KRange kr = k_range<Cfg, SPLIT>(p, pid, it, nk);
+      const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, it, nk);
       for (int k = kr.k_begin; k < kr.k_end; ++k) {
         __syncthreads();  // previous step's readers are done with the stage
         load_slab_generic<Cfg>(p, c_it, lds, k, tid);

@@ -221,34 +221,70 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   k.partial_stride = a.partials_slot_elems;
   k.status = a.status;
   k.timeout = a.spin_timeout_ticks ? a.spin_timeout_ticks : 200000000ull;  // 2 s at 100 MHz
-  if (a.split_k < 0) return hipErrorInvalidValue;
+  k.stream_k = 0;
+  if (a.split_k < 0 && a.split_k != IRIS_GEMM_SPLIT_STREAM_K) return hipErrorInvalidValue;
+  const int nk = (a.K + pick->bk - 1) / pick->bk;
   if (a.split_k != 1 && a.partials && a.locks) {
-    const int nk = (a.K + pick->bk - 1) / pick->bk;
     int cus = 0, dev = 0;
     const bool resident = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 && a.num_sms <= cus;
     const bool possible = resident && pick->splitk && pick->fn_split && k.sub_m == 1 && k.sub_n == 1 &&
                           a.partials_slot_elems >= (int64_t)pick->cm * pick->cn &&
                           (reinterpret_cast<uintptr_t>(a.partials) & 15) == 0 && (a.partials_slot_elems % 4) == 0;
-    if (a.split_k > 1) {
+    // Stream-K: every program takes the same number of K-steps (within one).
+    // A run of at least four steps keeps the parts of a tile few.
+    const int64_t steps = (int64_t)k.total_tiles * nk;
+    const int run = (int)(steps / a.num_sms);
+    const bool stream_ok = possible && run >= 4 && steps < ((int64_t)1 << 30) && (nk + run - 1) / run + 1 <= 32;
+    if (a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
+      if (!stream_ok) return hipErrorInvalidValue;
+      k.stream_k = 1;
+    } else if (a.split_k > 1) {
       if (!possible || a.split_k > nk || a.split_k > 64 || (int64_t)k.total_tiles * a.split_k > a.num_sms)
         return hipErrorInvalidValue;
       k.split_k = a.split_k;
-    } else if (possible && k.total_tiles * 2 <= a.num_sms && nk >= 32) {
-      // The hand-over of partials costs about as much as ten K-steps of a
-      // small tile, so only long K loops are split: as many parts as there
-      // are idle programs, at least four K-steps each.
-      int sk = a.num_sms / k.total_tiles;
-      if (sk > nk / 4) sk = nk / 4;
-      if (sk > 16) sk = 16;
-      if (sk > 1) k.split_k = sk;
+    } else if (possible) {
+      // K-steps a program walks through, unsplit
+      const int rounds = (k.total_tiles + a.num_sms - 1) / a.num_sms;
+      int walk = rounds * nk;
+      if (k.total_tiles * 2 <= a.num_sms && nk >= 32) {
+        // The hand-over of partials costs about as much as ten K-steps of a
+        // small tile, so only long K loops are split: as many parts as there
+        // are idle programs, at least four K-steps each.
+        int sk = a.num_sms / k.total_tiles;
+        if (sk > nk / 4) sk = nk / 4;
+        if (sk > 16) sk = 16;
+        if (sk > 1) {
+          k.split_k = sk;
+          walk = (nk + sk - 1) / sk;
+        }
+      }
+      // Stream-K when it shortens that walk by 15 % or more.  With runs of at
+      // least a tile's length a tile spans two runs and the second hands its
+      // part over first thing, long before the owner asks: nothing is lost.
+      // With shorter runs the owner waits for programs that finish when it
+      // does, and more CUs pull operands at once; measured on the decoder
+      // shapes that pays when the walk is long and at least 45 % shorter than
+      // the unsplit one (132 tiles of 64 steps on 256 programs: -17 %; 176
+      // tiles: +9 %; 22-step tiles: +6 to +20 %).
+      const bool hidden = run >= nk;
+      if (stream_ok && nk >= 16 && run >= 8 && (int64_t)(run + 1) * 20 <= (int64_t)walk * 17 &&
+          (hidden || (nk >= 32 && (int64_t)(run + 1) * 20 <= (int64_t)rounds * nk * 11))) {
+        k.stream_k = 1;
+        k.split_k = 1;
+      }
     }
-  } else if (a.split_k > 1) {
+  } else if (a.split_k > 1 || a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
     return hipErrorInvalidValue;  // forced, but no workspace
   }
   if (k.split_k > 1) {
-    const int nk = (a.K + pick->bk - 1) / pick->bk;
     k.split_q = nk / k.split_k;
     k.split_r = nk % k.split_k;
+  }
+  if (k.stream_k) {
+    const int64_t steps = (int64_t)k.total_tiles * nk;
+    k.split_q = (int)(steps / a.num_sms);
+    k.split_r = (int)(steps % a.num_sms);
+    return hipSuccess;  // (every program has a run: the reference's XCD remap stays)
   }
   // Fewer (tile, part) items than programs: deal them to the XCDs evenly, in
   // consecutive runs, instead of filling the first XCDs and idling the rest.
@@ -318,7 +354,7 @@ extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
     if (err != hipSuccess) return err;
   } else if (plan.entry) {
     const GemmKernelEntry* e = plan.entry;
-    const GemmKernelFn fn = plan.k.split_k > 1 ? e->fn_split : e->fn;
+    const GemmKernelFn fn = (plan.k.split_k > 1 || plan.k.stream_k) ? e->fn_split : e->fn;
     if (e->lds_bytes > 64 * 1024) {
       err = ensure_lds(fn, e->lds_bytes);
       if (err != hipSuccess) return err;
@@ -346,7 +382,7 @@ extern "C" int iris_gemm_split_k(const iris_gemm_args* args, int* split_k) {
   Plan plan;
   hipError_t err = make_plan(*args, &plan);
   if (err != hipSuccess) return err;
-  *split_k = plan.entry && !plan.skinny ? plan.k.split_k : 1;
+  *split_k = plan.entry && !plan.skinny ? (plan.k.stream_k ? IRIS_GEMM_SPLIT_STREAM_K : plan.k.split_k) : 1;
   return hipSuccess;
 }
 
@@ -380,6 +416,7 @@ extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t
   Plan plan;
   hipError_t err = make_plan(*args, &plan);
   if (err != hipSuccess) return err;
-  std::snprintf(buf, len, "%s", plan.skinny ? "few_rows_16xN" : plan.entry ? plan.entry->name : "");
+  std::snprintf(buf, len, "%s%s", plan.skinny ? "few_rows_16xN" : plan.entry ? plan.entry->name : "",
+                plan.entry && plan.k.stream_k ? "+stream_k" : "");
   return hipSuccess;
 }

@@ -27,6 +27,7 @@ from ._native import (
     SCOPE_SYSTEM,
     VARIANT_FEW_ROWS,
     VARIANT_PERSISTENT,
+    SPLIT_STREAM_K,
 )
 
 __all__ = [
@@ -213,8 +214,8 @@ def _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_s
             raise ValueError("partials need one slot per program")
         args.partials = _ptr(partials)
         args.partials_slot_elems = partials.shape[1]
-    elif split_k > 1:
-        raise ValueError("split_k > 1 needs the partials and locks workspace")
+    if partials is None and (split_k > 1 or split_k == SPLIT_STREAM_K):
+        raise ValueError("a forced split of K needs the partials and locks workspace")
     args.split_k = split_k
     return args
 
@@ -227,7 +228,9 @@ def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size,
 
     ``partials`` / ``locks`` are the wrappers' ``P`` and ``locks`` buffers
     (matmul_wrapper.py:29-31): with them, a launch with far fewer tiles than
-    programs splits each tile's K range over several programs (``split_k`` 0:
+    programs splits each tile's K range over several programs, and a launch
+    whose last round of tiles would leave many programs idle is cut into equal
+    runs of K-steps (stream-K, ``split_k=SPLIT_STREAM_K`` to insist) (``split_k`` 0:
     the launcher decides, 1: never, n: exactly n).
 
     The kernel launch of the reference wrappers (matmul_wrapper.py:109-150).

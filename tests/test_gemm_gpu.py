@@ -468,6 +468,123 @@ def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
                         partials=shmem.zeros((256, 256 * 256), dtype=torch.float32), locks=locks, split_k=2)
 
 
+STREAM_K_CASES = [
+    # M, N, K, BLK_M, BLK_N, grid, dtype
+    (2048, 1376, 1024, 128, 128, 256, torch.bfloat16),  # 176 tiles x 16 steps on 256 programs: runs of 11
+    (512, 768, 2048, 128, 128, 16, torch.bfloat16),     # 24 x 32 steps on 16 programs: tail, whole tile, head
+    (300, 200, 1376, 64, 64, 24, torch.float16),        # ragged M, N and K; 20 x 22 steps = 24 runs of 18 or 19
+    (256, 320, 4096, 256, 64, 8, torch.bfloat16),       # 5 x 64 steps on 8 programs
+    (64, 128, 8192, 64, 64, 16, torch.bfloat16),        # 2 tiles, 8 runs each: an owner and seven followers
+    (128, 128, 512, 64, 64, 4, torch.float16),          # runs that end exactly at tile boundaries
+]
+
+
+@pytest.mark.parametrize("M,N,K,BM,BN,grid,dtype", STREAM_K_CASES)
+def test_stream_k_all_scatter(shmem, M, N, K, BM, BN, grid, dtype):
+    """The launch's K-steps cut into equal runs that cross tile boundaries:
+    the program that holds a tile's first step owns it and adds what the
+    programs after it hand over.  Twice in a row: the locks are left re-armed."""
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    partials, locks = split_workspace(shmem, grid, BM, BN)
+    args = (a, b, None, cg, flags, None, 0, 1, grid, BM, BN, 64, 2, ops.EPI_ALL_SCATTER)
+    kw = dict(partials=partials, locks=locks, split_k=ops.SPLIT_STREAM_K, num_xcds=ops.default_num_xcds(256, grid))
+    assert ops.gemm_split_k(*args, **kw) == ops.SPLIT_STREAM_K
+    assert ops.gemm_plan_name(*args, **kw).endswith("+stream_k")
+    want = O.shard_gemm(A, B, dtype)
+    for launch in (1, 2):
+        cg.zero_()
+        ops.gemm_launch(*args, **kw)
+        torch.cuda.synchronize()
+        check_close(cg, want, f"launch {launch}")
+        assert flags.cpu().tolist() == [launch] * total
+        assert int(locks.abs().max().item()) == 0
+
+
+def test_stream_k_is_chosen_when_the_last_round_of_tiles_is_thin(shmem):
+    dtype = torch.bfloat16
+    A, B = make_ab(1024, 1376, 2048, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((1024, 1376), dtype=dtype)
+    flags = shmem.zeros((128,), dtype=torch.int32)
+    partials, locks = split_workspace(shmem, 256, 128, 128)
+
+    def choice(grid, BM, BN, **kw):
+        return ops.gemm_split_k(a, b, None, cg, flags, None, 0, 1, grid, BM, BN, 64, 4, ops.EPI_ALL_SCATTER,
+                                partials=partials, locks=locks, **kw)
+
+    assert choice(256, 128, 128) == ops.SPLIT_STREAM_K       # 88 tiles on 256 programs
+    assert choice(64, 128, 128) == ops.SPLIT_STREAM_K        # 88 tiles on 64 programs: 1.4 rounds
+    assert choice(88, 128, 128) == 1                         # one tile each
+    assert choice(44, 128, 128) == 1                         # two rounds, both full
+    assert choice(256, 128, 128, split_k=1) == 1
+    assert choice(256, 256, 256) == 1                        # a tile whose kernel has no split build
+    ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 256, 128, 128, 64, 4, ops.EPI_ALL_SCATTER, partials=partials,
+                    locks=locks)
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, dtype))
+    assert flags.cpu().tolist()[:88] == [1] * 88 and int(locks.abs().max().item()) == 0
+    with pytest.raises(ValueError):  # no workspace
+        ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 256, 128, 128, 64, 4, ops.EPI_ALL_SCATTER,
+                        split_k=ops.SPLIT_STREAM_K)
+    with pytest.raises(ValueError):  # runs shorter than four steps
+        ops.gemm_launch(a[:, :128], b[:128, :], None, cg, flags, None, 0, 1, 256, 128, 128, 64, 4,
+                        ops.EPI_ALL_SCATTER, partials=partials, locks=locks, split_k=ops.SPLIT_STREAM_K)
+
+
+def test_stream_k_with_the_other_epilogues_and_virtual_ranks(shmem):
+    """Atomic accumulate and the one-shot producer behind stream-K runs."""
+    dtype = torch.bfloat16
+    ws = 4
+    M, N, K = 192, 320, 4 * 768
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    hb = shmem.get_heap_bases()
+    shards = O.k_shards(A, B, ws)
+    kk = K // ws
+    grid, BM, BN = 16, 64, 64
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    partials, locks = split_workspace(shmem, grid, BM, BN)
+    # 08: every rank adds its shard product into every rank's fp32 C
+    cg = shmem.zeros((M, N), dtype=torch.float32)
+    for r in range(ws):
+        shmem.on_rank(cg, r).zero_()
+    for r in range(ws):
+        ops.gemm_launch(a[:, r * kk:(r + 1) * kk], b[r * kk:(r + 1) * kk, :], None, shmem.on_rank(cg, r), None, hb, r,
+                        ws, grid, BM, BN, 64, 4, ops.EPI_ATOMIC_ADD, partials=shmem.on_rank(partials, r),
+                        locks=shmem.on_rank(locks, r), split_k=ops.SPLIT_STREAM_K)
+    torch.cuda.synchronize()
+    want = O.atomics_all_reduce(shards)
+    for r in range(ws):
+        check_close(shmem.on_rank(cg, r), want, f"atomic, rank {r}")
+    # 09: producers, then the reduce
+    part = shmem.zeros((M, N), dtype=torch.float32)
+    out = shmem.zeros((M, N), dtype=dtype)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    for r in range(ws):
+        for t in (part, out, flags):
+            shmem.on_rank(t, r).zero_()
+    for r in range(ws):
+        ops.gemm_launch(a[:, r * kk:(r + 1) * kk], b[r * kk:(r + 1) * kk, :], shmem.on_rank(part, r),
+                        shmem.on_rank(out, r), shmem.on_rank(flags, r), hb, r, ws, grid, BM, BN, 64, 6,
+                        ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=shmem.on_rank(partials, r),
+                        locks=shmem.on_rank(locks, r), split_k=ops.SPLIT_STREAM_K)
+    torch.cuda.synchronize()
+    for r in range(ws):
+        assert shmem.on_rank(flags, r).cpu().tolist() == [ws - 1] * total
+        assert not shmem.on_rank(locks, r).any()
+    for r in range(ws):
+        ops.one_shot_reduce(shmem.on_rank(part, r), shmem.on_rank(out, r), shmem.on_rank(flags, r), hb, r, ws, BM,
+                            BN, 6)
+    torch.cuda.synchronize()
+    want = O.one_shot_all_reduce(shards, torch.float32, dtype)
+    for r in range(ws):
+        check_close(shmem.on_rank(out, r), want, f"one-shot, rank {r}")
+
+
 def test_split_k_with_the_other_epilogues_and_virtual_ranks(shmem):
     """Atomic accumulate and the one-shot producer behind a split K loop."""
     dtype = torch.bfloat16
