@@ -236,7 +236,7 @@ def run_atomic(args):
     def step():
         for i in range(shards):
             ops.gemm_launch(a_full[:, i * ks:(i + 1) * ks], bt_full[:, i * ks:(i + 1) * ks].T, None, c, None, hb, 0, 1,
-                            grid, blk_m, blk_n, 64, 6, ops.EPI_ATOMIC_ADD, num_xcds=num_xcds)
+                            grid, blk_m, blk_n, 64, 6, ops.EPI_ATOMIC_ADD, num_xcds=num_xcds, variant=args.variant)
 
     step()
     torch.cuda.synchronize()

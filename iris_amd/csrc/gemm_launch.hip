@@ -196,6 +196,11 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
       if (a.block_m % e.cm != 0 || a.block_n % e.cn != 0) continue;
       if (e.cm > 64 && e.cm >= 2 * a.M) continue;
       if (e.cn > 64 && e.cn >= 2 * a.N) continue;
+      // An atomic epilogue is bound by the chip's atomic rate (329 G fp32
+      // adds a second, 51 us for 4096 x 4096), and while a program walks its
+      // K loop it sends none: with two half tiles per logical tile the
+      // second's K loop runs while the first's atomics drain (-7 % per launch).
+      if ((op == OP_ATOMIC32 || op == OP_ATOMIC16) && e.cm * e.cn > 256 * 128) continue;
       pick = &e;
     }
     // otherwise the smallest tile that fits, with masked sub-tiles
