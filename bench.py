@@ -50,6 +50,8 @@ def parse():
                          "~10 ms, which a short run would measure instead of the steady state")
     ap.add_argument("--variant", type=int, default=0, help="GEMM kernel tuning variant (0 = default)")
     ap.add_argument("--reduce-variant", type=int, default=0)
+    ap.add_argument("--decoder-m", default="1,16,128,512,2048",
+                    help="decoder workload: the row counts to run (comma-separated)")
     ap.add_argument("--gsize_m", type=int, default=GSIZE_M)
     ap.add_argument("--no-reduce", action="store_true", help="skip the reduce-phase measurement")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -273,7 +275,7 @@ def run_decoder(args):
     hb = shmem.get_heap_bases()
     g = torch.Generator().manual_seed(123)
     rows = []
-    for Mt in (1, 16, 128, 512, 2048):
+    for Mt in [int(t) for t in args.decoder_m.split(",")]:
         off = shmem.heap_offset
         x = shmem.zeros((Mt, hidden), dtype=torch.bfloat16)
         x.copy_((torch.randn(Mt, hidden, generator=g) * 0.02).to(torch.bfloat16))
