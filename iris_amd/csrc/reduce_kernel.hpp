@@ -29,6 +29,8 @@ struct ReduceKArgs {
   int sys, wait_flags;
   // row-band kernel: an item is `band_rows` rows x `band_vecs` 16-byte strips
   int band_rows, band_vecs, band_chunks, band_items;
+  // tile kernel: fetch the ranks' heap bases with vector loads (see there)
+  int pace;
 };
 
 // VE<DT>: elements in one 16-byte load of type DT.  A lane always moves 16
@@ -135,13 +137,17 @@ __global__ __launch_bounds__(256) void reduce_tiles_vec_kernel(const ReduceKArgs
     const int64_t in0 = ((int64_t)m0 * p.scm + n0) * IES;
     const __amdgpu_buffer_rsrc_t out_rs =
         tile_rsrc((const IRIS_GLOBAL char*)p.cg + ((int64_t)m0 * p.sgm + n0) * OES, out_bytes);
-    // The bases come through vector loads on purpose: the wait for the
-    // outstanding loads that such a load forces between the ranks' batches
-    // paces the tile walk, and measured 9% faster than scalar loads of them.
+    // With many tiles per program the bases come through vector loads on
+    // purpose: the wait for the outstanding loads that such a load forces
+    // between the ranks' batches paces the tile walk, and measured 9% faster
+    // than scalar loads of them.  A program with a single small tile has
+    // nothing to pace and eight round trips to lose: its bases come through
+    // scalar loads and all ranks' strips are in flight together.
     auto rank_rsrc = [&](int rk) __attribute__((always_inline)) {
-      const IRIS_GLOBAL char* b = (rk == p.cur_rank || !p.heap_bases)
-                                      ? (const IRIS_GLOBAL char*)p.c
-                                      : translate(p.c, cur_base, uniform_u64(p.heap_bases[rk]));
+      const IRIS_GLOBAL char* b = (const IRIS_GLOBAL char*)p.c;
+      if (rk != p.cur_rank && p.heap_bases)
+        b = translate(p.c, cur_base,
+                      p.pace ? uniform_u64(p.heap_bases[rk]) : uniform_u64(heap_base_at(p.heap_bases, rk)));
       return tile_rsrc(b + in0, in_bytes);
     };
 

@@ -147,6 +147,8 @@ extern "C" int iris_one_shot_reduce_launch(const iris_reduce_args* a, void* stre
     rows = fits && (a->variant == 7 ||
                     (a->variant == 0 && (int64_t)k.N * ies >= 16384 && k.band_items >= current_cu_count()));
   }
+  // (the tile kernel paces its walk only when a program has several tiles)
+  k.pace = k.total_tiles > grid ? 1 : 0;
   ReduceFn fn = vec ? pick(k.c_dt, k.cg_dt, k.ws, a->variant, k.sys != 0, rows) : nullptr;
   if (!fn) {
     fn = &reduce_tiles_generic_kernel;
