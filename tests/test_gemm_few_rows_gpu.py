@@ -17,10 +17,11 @@ pytestmark = pytest.mark.gpu
 FEW = "few_rows_16xN"
 
 
-def scatter(shmem, a, b, cg, flags, rank, ws, BM, BN, G, *, locks=None, variant=0, notify=True, grid=256):
+def scatter(shmem, a, b, cg, flags, rank, ws, BM, BN, G, *, locks=None, variant=0, notify=True, grid=256,
+            scope=ops.SCOPE_AGENT):
     args = (a, b, None, cg, flags, shmem.get_heap_bases(), rank, ws, grid, BM, BN, 64, G, ops.EPI_ALL_SCATTER)
     name = ops.gemm_plan_name(*args, notify=notify, locks=locks, partials=None, variant=variant)
-    ops.gemm_launch(*args, notify=notify, locks=locks, variant=variant)
+    ops.gemm_launch(*args, notify=notify, locks=locks, variant=variant, scope=scope)
     return name
 
 
@@ -72,8 +73,8 @@ def test_strided_operands_and_output(shmem):
     assert flags.cpu().tolist() == [1, 1]
 
 
-@pytest.mark.parametrize("ws", [2, 8])
-def test_scatter_virtual_ranks(shmem, ws):
+@pytest.mark.parametrize("ws,scope", [(2, ops.SCOPE_AGENT), (8, ops.SCOPE_AGENT), (3, ops.SCOPE_SYSTEM)])
+def test_scatter_virtual_ranks(shmem, ws, scope):
     """Rank r's [M, N/ws] block lands at column r*N/ws of c_global on every
     rank (wave w of a workgroup stores on rank w); every rank's flags count ws
     arrivals."""
@@ -93,7 +94,7 @@ def test_scatter_virtual_ranks(shmem, ws):
         shmem.on_rank(flags, r).zero_()
     for r in range(ws):
         assert scatter(shmem, a, bs[r], shmem.on_rank(cg, r), shmem.on_rank(flags, r), r, ws, BM, BN, G,
-                       locks=shmem.on_rank(locks, r)) == FEW
+                       locks=shmem.on_rank(locks, r), scope=scope) == FEW
     torch.cuda.synchronize()
     want = O.all_scatter(shards, dtype)
     for r in range(ws):
