@@ -161,7 +161,7 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
                           (a.locks && k.total_tiles <= a.num_sms);
     const bool ok = a.M <= SKINNY_ROWS && a.K > 0 && dma_ok && (op == OP_STORE16 || op == OP_STORE32) &&
                     a.block_m >= a.M && (a.block_n % SKINNY_COLS) == 0 && !a.mm_begin_timestamp &&
-                    !a.mm_end_timestamp && a.split_k <= 1 && counters &&
+                    !a.mm_end_timestamp && (a.split_k == 0 || a.split_k == 1) && counters &&
                     ((int64_t)SKINNY_ROWS * a.stride_am + a.K) * 2 < lim &&
                     ((int64_t)SKINNY_COLS * a.stride_bn + a.K) * 2 < lim;
     if (ok) {
