@@ -90,8 +90,8 @@ def test_scatter_virtual_ranks(shmem, ws, scope):
     flags = shmem.zeros((total,), dtype=torch.int32)
     locks = shmem.zeros((256,), dtype=torch.int32)
     for r in range(ws):
-        shmem.on_rank(cg, r).zero_()
-        shmem.on_rank(flags, r).zero_()
+        for t in (cg, flags, locks):  # (zeros() clears rank 0's copy only)
+            shmem.on_rank(t, r).zero_()
     for r in range(ws):
         assert scatter(shmem, a, bs[r], shmem.on_rank(cg, r), shmem.on_rank(flags, r), r, ws, BM, BN, G,
                        locks=shmem.on_rank(locks, r), scope=scope) == FEW

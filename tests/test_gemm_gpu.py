@@ -552,6 +552,7 @@ def test_stream_k_with_the_other_epilogues_and_virtual_ranks(shmem):
     cg = shmem.zeros((M, N), dtype=torch.float32)
     for r in range(ws):
         shmem.on_rank(cg, r).zero_()
+        shmem.on_rank(locks, r).zero_()  # (zeros() clears rank 0's copy only)
     for r in range(ws):
         ops.gemm_launch(a[:, r * kk:(r + 1) * kk], b[r * kk:(r + 1) * kk, :], None, shmem.on_rank(cg, r), None, hb, r,
                         ws, grid, BM, BN, 64, 4, ops.EPI_ATOMIC_ADD, partials=shmem.on_rank(partials, r),
