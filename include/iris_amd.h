@@ -99,9 +99,9 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 #define IRIS_STATUS_OK 0
 #define IRIS_STATUS_SPIN_TIMEOUT 1 /* a flag wait gave up; that tile was not reduced */
 
-/* Special values of iris_gemm_args.variant.  A launch with at most 16 rows of
+/* Special values of iris_gemm_args.variant.  A launch with at most 32 rows of
  * A whose operands are K-contiguous normally takes a kernel of its own that
- * streams B once (one workgroup per 16 columns of C, no LDS staging);
+ * streams B (one workgroup per 16 rows x 16 columns of C, all fetches in flight);
  * FEW_ROWS insists on it (hipErrorInvalidValue when the launch does not
  * qualify), PERSISTENT keeps the default choice among the persistent kernels.
  * The reference has one Triton kernel for every M (gemm_all_scatter.py:95). */

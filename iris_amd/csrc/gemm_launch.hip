@@ -42,7 +42,7 @@ struct Plan {
   int fused_reduce = 0;  // ONE_SHOT with the CONSUME phase: follow with the reduce kernel
   // the few-rows kernel instead of a table entry, one workgroup per 16 columns
   GemmKernelFn skinny = nullptr;
-  int skinny_grid = 0, skinny_lds = 0;
+  int skinny_grid = 0, skinny_grid_y = 1, skinny_lds = 0;
 };
 
 int dbg() {
@@ -152,25 +152,37 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
     return ((int64_t)e.cm * a.stride_am + a.K) * 2 < lim && ((int64_t)e.cn * a.stride_bn + a.K) * 2 < lim;
   };
 
-  // At most 16 rows: the product is a stream over B, and the kernel built for
+  // A few rows: the product is a stream over B, and the kernel built for
   // that takes it when the operands allow the 16-byte fetches, the logical
-  // tile covers every row, and the tiles' arrival counters have a home.
+  // tile covers every row, the tiles' arrival counters have a home, and (with
+  // more than 16 rows: two workgroups per 16 columns) every workgroup finds
+  // a place on the device at once, so that B comes from HBM once.
   if (a.variant == 0 || a.variant == IRIS_GEMM_VARIANT_FEW_ROWS) {
     const int64_t lim = (int64_t)1 << 31;
-    const bool counters = a.block_n <= SKINNY_COLS || a.N <= SKINNY_COLS || k.flag_mode == 0 ||
+    const int m_blocks = (a.M + SKINNY_ROWS - 1) / SKINNY_ROWS;
+    const int n_blocks = (a.N + SKINNY_COLS - 1) / SKINNY_COLS;
+    const int per_wave = ((a.K + 63) / 64 + SKINNY_WAVES - 1) / SKINNY_WAVES;
+    const int un = per_wave <= 2 ? 2 : per_wave <= 4 ? 4 : 8;
+    const bool counters = (m_blocks == 1 && (a.block_n <= SKINNY_COLS || a.N <= SKINNY_COLS)) || k.flag_mode == 0 ||
                           (a.locks && k.total_tiles <= a.num_sms);
-    const bool ok = a.M <= SKINNY_ROWS && a.K > 0 && dma_ok && (op == OP_STORE16 || op == OP_STORE32) &&
+    bool room = true;
+    if (m_blocks > 1) {
+      int cus = 0, dev = 0;
+      const int per_cu = 160 * 1024 / skinny_lds_bytes(un) > 4 ? 4 : 160 * 1024 / skinny_lds_bytes(un);
+      room = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 &&
+             (int64_t)m_blocks * n_blocks <= (int64_t)cus * per_cu;
+    }
+    const bool ok = a.M <= SKINNY_MAX_ROWS && room && a.K > 0 && dma_ok && (op == OP_STORE16 || op == OP_STORE32) &&
                     a.block_m >= a.M && (a.block_n % SKINNY_COLS) == 0 && !a.mm_begin_timestamp &&
                     !a.mm_end_timestamp && (a.split_k == 0 || a.split_k == 1) && counters &&
                     ((int64_t)SKINNY_ROWS * a.stride_am + a.K) * 2 < lim &&
                     ((int64_t)SKINNY_COLS * a.stride_bn + a.K) * 2 < lim;
     if (ok) {
-      // fetches in flight per wave: enough for the whole K range, 8 blocks at most
-      const int per_wave = ((a.K + 63) / 64 + SKINNY_WAVES - 1) / SKINNY_WAVES;
-      const int un = per_wave <= 2 ? 2 : per_wave <= 4 ? 4 : 8;
+      // (un: fetches in flight per wave, enough for the whole K range, 8 blocks at most)
       plan->skinny = gemm_skinny_kernel_for(a.ab_dtype, op, un);
       plan->skinny_lds = skinny_lds_bytes(un);
-      plan->skinny_grid = (a.N + SKINNY_COLS - 1) / SKINNY_COLS;
+      plan->skinny_grid = n_blocks;
+      plan->skinny_grid_y = m_blocks;
       k.split_k = 1;
       k.locks = a.locks;
       if (plan->skinny) return hipSuccess;
@@ -348,13 +360,14 @@ extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (plan.skinny) {
     if (dbg())
-      std::fprintf(stderr, "[iris_amd] gemm few-rows M=%d N=%d K=%d tiles=%d grid=%d\n", plan.k.M, plan.k.N, plan.k.K,
-                   plan.k.total_tiles, plan.skinny_grid);
+      std::fprintf(stderr, "[iris_amd] gemm few-rows M=%d N=%d K=%d tiles=%d grid=%dx%d\n", plan.k.M, plan.k.N, plan.k.K,
+                   plan.k.total_tiles, plan.skinny_grid, plan.skinny_grid_y);
     if (plan.skinny_lds > 64 * 1024) {
       err = ensure_lds(plan.skinny, plan.skinny_lds);
       if (err != hipSuccess) return err;
     }
-    hipLaunchKernelGGL(plan.skinny, dim3(plan.skinny_grid), dim3(SKINNY_THREADS), plan.skinny_lds, s, plan.k);
+    hipLaunchKernelGGL(plan.skinny, dim3(plan.skinny_grid, plan.skinny_grid_y), dim3(SKINNY_THREADS), plan.skinny_lds, s,
+                       plan.k);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
   } else if (plan.entry) {

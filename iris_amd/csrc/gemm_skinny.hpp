@@ -1,4 +1,4 @@
-// Shard GEMM for at most 16 rows of A (decode-time batches): C[M,N] = A[M,K] B[K,N]
+// Shard GEMM for a few rows of A (decode-time batches, 16 rows a workgroup): C[M,N] = A[M,K] B[K,N]
 // with the store epilogues of the persistent kernel (gemm_all_scatter.py:209-251,
 // gemm_one_shot_all_reduce.py:197-218).
 //
@@ -18,8 +18,8 @@
 // The eight partial 16x16 accumulators meet in LDS; wave w then stores the
 // sum on destination rank w, w+8, ...
 //
-// A logical tile (BLOCK_SIZE_M x BLOCK_SIZE_N, one flag) spans several such
-// workgroups.  They count their arrivals in locks[tile_id]; the last one to
+// A logical tile (BLOCK_SIZE_M x BLOCK_SIZE_N, one flag; BLOCK_SIZE_M covers
+// every row) spans several such workgroups.  They count their arrivals in locks[tile_id]; the last one to
 // arrive re-arms the counter and publishes the tile's flag.
 #pragma once
 
@@ -27,7 +27,8 @@
 
 namespace iris_amd {
 
-constexpr int SKINNY_ROWS = 16;    // rows of A a launch can take
+constexpr int SKINNY_ROWS = 16;    // rows of A per workgroup (blockIdx.y counts blocks of them)
+constexpr int SKINNY_MAX_ROWS = 32;  // rows of A a launch can take: beyond, B is re-read too often
 constexpr int SKINNY_COLS = 16;    // columns of C per workgroup
 constexpr int SKINNY_WAVES = 8;
 constexpr int SKINNY_THREADS = SKINNY_WAVES * 64;
@@ -51,6 +52,7 @@ gemm_skinny_kernel(const GemmKArgs p) {
   const int lane = tid & 63;
   const int lr = lane & 15, lq = lane >> 4;
   const int n0 = blockIdx.x * SKINNY_COLS;
+  const int m0 = blockIdx.y * SKINNY_ROWS;
   IRIS_LDS char* wb = lds + SKINNY_RED_BYTES + wave * (UN * SKINNY_BLOCK_BYTES);
 
   // Rows past the edge of either operand lie past the end of its buffer
@@ -58,8 +60,9 @@ gemm_skinny_kernel(const GemmKArgs p) {
   const int rows_b = min(SKINNY_COLS, p.N - n0);
   const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(p.b + (int64_t)n0 * p.sbn * 2), 0, (int)((((int64_t)rows_b - 1) * p.sbn + p.K) * 2), 0x00020000);
+  const int rows_a = min(SKINNY_ROWS, p.M - m0);
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)p.a, 0, (int)((((int64_t)p.M - 1) * p.sam + p.K) * 2), 0x00020000);
+      (void*)(p.a + (int64_t)m0 * p.sam * 2), 0, (int)((((int64_t)rows_a - 1) * p.sam + p.K) * 2), 0x00020000);
   // B: lane l of fetch j of a block brings row 8j + l/8 and lands at byte
   // l*16 of the fetch's 1 KiB, i.e. at physical chunk l%8 of that row; the
   // chunk of the row it must bring there is (l%8) ^ (row/2 % 8).
@@ -116,7 +119,7 @@ gemm_skinny_kernel(const GemmKArgs p) {
 
   const int r_begin = p.dest_all ? 0 : p.cur_rank;
   const int r_end = p.dest_all ? p.ws : p.cur_rank + 1;
-  const int m = lr, n = n0 + lq * 4;
+  const int m = m0 + lr, n = n0 + lq * 4;
   if (r_begin + wave < r_end && m < p.M && n < p.N) {
     f32x4 s = red[lane];
 #pragma unroll
@@ -161,7 +164,7 @@ gemm_skinny_kernel(const GemmKArgs p) {
     const int pid_n = n0 / p.BN;
     const int tile_id = tile_id_of(0, pid_n, p.num_pid_m, p.num_pid_n, p.G);
     const int cols = min(p.N, (pid_n + 1) * p.BN) - pid_n * p.BN;
-    const int parts = (cols + SKINNY_COLS - 1) / SKINNY_COLS;
+    const int parts = ((cols + SKINNY_COLS - 1) / SKINNY_COLS) * gridDim.y;
     bool last = true;
     if (parts > 1) {
       IRIS_GLOBAL int32_t* cnt = (IRIS_GLOBAL int32_t*)(p.locks + tile_id);

@@ -1,5 +1,5 @@
-"""Parity of the few-rows shard GEMM (at most 16 rows of A, one workgroup per
-16 columns of C) against the CPU oracle, through the C-ABI.
+"""Parity of the few-rows shard GEMM (at most 32 rows of A, one workgroup per
+16 rows x 16 columns of C) against the CPU oracle, through the C-ABI.
 
 Same bar as the persistent kernel: values rtol 1e-2 / atol 1e-2 against the
 fp32-accumulated oracle, flags and arrival counters bit-exact.
@@ -35,6 +35,9 @@ CASES = [
     (16, 16, 64, 16, 16, 1, torch.float16),
     (5, 272, 9000, 32, 48, 3, torch.bfloat16),      # K range that takes a wave two rounds of fetches
     (12, 2048, 640, 256, 128, 4, torch.float16),
+    (17, 1376, 4096, 64, 64, 4, torch.bfloat16),    # two blocks of rows, the second with one row
+    (32, 4096, 1376, 32, 128, 6, torch.bfloat16),
+    (20, 50, 72, 32, 16, 2, torch.float16),         # one block of columns per flag, two of rows
 ]
 
 
@@ -78,7 +81,7 @@ def test_scatter_virtual_ranks(shmem, ws, scope):
     """Rank r's [M, N/ws] block lands at column r*N/ws of c_global on every
     rank (wave w of a workgroup stores on rank w); every rank's flags count ws
     arrivals."""
-    M, K, BM, BN, G, dtype = 16, 512, 64, 64, 4, torch.bfloat16
+    M, K, BM, BN, G, dtype = (16 if ws != 2 else 27), 512, 64, 64, 4, torch.bfloat16
     N = 176 * ws
     A, B = make_ab(M, N, K, dtype)
     shards = O.n_shards(A, B, ws)
@@ -166,9 +169,12 @@ def test_choice_of_kernel(shmem):
     # a logical tile that does not cover the rows, or is no multiple of 16 columns
     assert plan(a, b, cg, 8, 64, locks=locks) != FEW
     assert plan(a, b, cg, 64, 40, locks=locks) != FEW
-    # more than 16 rows
-    A2, B2 = make_ab(17, 256, 128, dtype)
-    a2, cg2 = to_heap(shmem, A2), shmem.zeros((17, 256), dtype=dtype)
+    # up to 32 rows in blocks of 16; no more
+    A1, _ = make_ab(32, 256, 128, dtype)
+    assert plan(to_heap(shmem, A1), b, shmem.zeros((32, 256), dtype=dtype), 64, 64, locks=locks) == FEW
+    assert plan(to_heap(shmem, A1), b, shmem.zeros((32, 256), dtype=dtype), 32, 16) != FEW  # two workgroups a flag
+    A2, B2 = make_ab(33, 256, 128, dtype)
+    a2, cg2 = to_heap(shmem, A2), shmem.zeros((33, 256), dtype=dtype)
     assert plan(a2, b, cg2, 64, 64, locks=locks) != FEW
     with pytest.raises(ValueError):
         plan(a2, b, cg2, 64, 64, locks=locks, variant=ops.VARIANT_FEW_ROWS)
