@@ -144,6 +144,38 @@ def test_one_shot_producer_and_reduce(shmem, pdtype):
         assert not shmem.on_rank(flags, r).any()
 
 
+@pytest.mark.parametrize("ws", [1, 4])
+def test_one_shot_fused_phase(shmem, ws):
+    """PHASE_FUSED: the few-rows producer and the reduce kernel behind it on
+    the same stream.  With one GPU playing every rank the other ranks' partials
+    and signals are put in place first, then the last rank runs fused."""
+    M, N, BM, BN, G, dtype = 9, 272, 16, 64, 3, torch.bfloat16
+    K = 192 * ws
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    shards = O.k_shards(A, B, ws)
+    ah, bh = to_heap(shmem, A), to_heap(shmem, B)
+    kk = K // ws
+    part = shmem.zeros((M, N), dtype=torch.float32)
+    out = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(N, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    locks = shmem.zeros((256,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+    for r in range(ws):
+        for t in (part, out, flags, locks):
+            shmem.on_rank(t, r).zero_()
+    last = ws - 1
+    for r in range(ws):
+        args = (ah[:, r * kk:(r + 1) * kk], bh[r * kk:(r + 1) * kk, :], shmem.on_rank(part, r), shmem.on_rank(out, r),
+                shmem.on_rank(flags, r), hb, r, ws, 256, BM, BN, 64, G, ops.EPI_ONE_SHOT)
+        kw = dict(phase=ops.PHASE_FUSED if r == last else ops.PHASE_PRODUCE, locks=shmem.on_rank(locks, r))
+        assert ops.gemm_plan_name(*args, **kw) == FEW
+        ops.gemm_launch(*args, **kw)
+    torch.cuda.synchronize()
+    check_close(shmem.on_rank(out, last), O.one_shot_all_reduce(shards, torch.float32, dtype), "fused result")
+    assert not shmem.on_rank(flags, last).any()  # consumed
+
+
 def test_choice_of_kernel(shmem):
     dtype = torch.bfloat16
     A, B = make_ab(16, 256, 128, dtype)

@@ -476,6 +476,7 @@ STREAM_K_CASES = [
     (256, 320, 4096, 256, 64, 8, torch.bfloat16),       # 5 x 64 steps on 8 programs
     (64, 128, 8192, 64, 64, 16, torch.bfloat16),        # 2 tiles, 8 runs each: an owner and seven followers
     (128, 128, 512, 64, 64, 4, torch.float16),          # runs that end exactly at tile boundaries
+    (256, 384, 512, 64, 64, 5, torch.bfloat16),         # 24 x 8 steps on 5 programs: runs of four and five tiles
 ]
 
 
