@@ -243,6 +243,18 @@ void iris_tile_map_host(int32_t tile_id, int32_t M, int32_t N, int32_t block_m, 
                         int32_t group_size_m, int32_t* pid_m, int32_t* pid_n);
 
 /*
+ * The stream-K schedule exactly as the kernels compute it (the same source,
+ * compiled for the host), for checking it without a GPU: the items of program
+ * `pid` when `total_tiles` tiles of `k_steps` K-steps each are cut into
+ * `num_programs` runs.  items is int32[cap][4] = (tile, first K-step, end
+ * K-step, parts), parts being the number of programs that share the tile when
+ * this program owns it (its run holds the tile's first step) and 0 when it
+ * hands its part over; *n_items is the number of items of the run.
+ */
+int iris_stream_k_schedule_host(int32_t total_tiles, int32_t k_steps, int32_t num_programs, int32_t pid,
+                                int32_t* items, int32_t cap, int32_t* n_items);
+
+/*
  * Measurement aid; no counterpart in the reference.  `num_groups` workgroups of
  * 8 waves each run `iters` rounds of 16 v_mfma_f32_16x16x32 (ab_dtype: F16 or
  * BF16) per wave on operands read once from `operands` (64 KiB, 16-byte

@@ -162,22 +162,22 @@ struct KRange {
 struct StreamRun {
   int tile0, k0, g1;
 };
-__device__ inline int stream_len(const GemmKArgs& p, int pid) { return p.split_q + (pid < p.split_r ? 1 : 0); }
-__device__ inline StreamRun stream_run(const GemmKArgs& p, int pid, int nk) {
+__host__ __device__ inline int stream_len(const GemmKArgs& p, int pid) { return p.split_q + (pid < p.split_r ? 1 : 0); }
+__host__ __device__ inline StreamRun stream_run(const GemmKArgs& p, int pid, int nk) {
   StreamRun r;
-  const int g0 = pid * p.split_q + min(pid, p.split_r);
+  const int g0 = pid * p.split_q + (pid < p.split_r ? pid : p.split_r);
   r.g1 = g0 + stream_len(p, pid);
   r.tile0 = nk > 0 ? g0 / nk : 0;
   r.k0 = g0 - r.tile0 * nk;
   return r;
 }
 // Items (tiles touched) of the run.
-__device__ inline int stream_items(const StreamRun& r, int nk) {
+__host__ __device__ inline int stream_items(const StreamRun& r, int nk) {
   return r.g1 > r.tile0 * nk + r.k0 ? (r.g1 - 1) / nk - r.tile0 + 1 : 0;
 }
 // Parts of a tile whose owner, program `pid`, stops at step k_end: itself and
 // the programs that hold the rest (each run is at least one step long).
-__device__ inline int stream_parts(const GemmKArgs& p, int pid, int k_end, int nk) {
+__host__ __device__ inline int stream_parts(const GemmKArgs& p, int pid, int k_end, int nk) {
   int parts = 1;
   for (int rem = nk - k_end, q = pid + 1; rem > 0; ++q, ++parts) rem -= stream_len(p, q);
   return parts;

@@ -438,3 +438,28 @@ extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t
                 plan.entry && plan.k.stream_k ? "+stream_k" : "");
   return hipSuccess;
 }
+
+extern "C" int iris_stream_k_schedule_host(int32_t total_tiles, int32_t k_steps, int32_t num_programs, int32_t pid,
+                                           int32_t* items, int32_t cap, int32_t* n_items) {
+  if (total_tiles <= 0 || k_steps <= 0 || num_programs <= 0 || pid < 0 || pid >= num_programs || !n_items ||
+      (int64_t)total_tiles * k_steps >= ((int64_t)1 << 30))
+    return hipErrorInvalidValue;
+  GemmKArgs k{};
+  const int64_t steps = (int64_t)total_tiles * k_steps;
+  k.split_q = (int)(steps / num_programs);
+  k.split_r = (int)(steps % num_programs);
+  if (k.split_q < 1) return hipErrorInvalidValue;  // the kernel is never launched with empty runs
+  const StreamRun sr = stream_run(k, pid, k_steps);
+  const int n = stream_items(sr, k_steps);
+  *n_items = n;
+  for (int i = 0; i < n && i < cap && items; ++i) {
+    // the kernel's k_range for a split build, and the owner's count of parts
+    const int k_begin = i == 0 ? sr.k0 : 0;
+    const int k_end = sr.g1 - (sr.tile0 + i) * k_steps < k_steps ? sr.g1 - (sr.tile0 + i) * k_steps : k_steps;
+    items[4 * i + 0] = sr.tile0 + i;
+    items[4 * i + 1] = k_begin;
+    items[4 * i + 2] = k_end;
+    items[4 * i + 3] = k_begin == 0 ? stream_parts(k, pid, k_end, k_steps) : 0;
+  }
+  return hipSuccess;
+}

@@ -35,6 +35,7 @@ __all__ = [
     "gemm_kernel_info",
     "gemm_split_k",
     "gemm_plan_name",
+    "stream_k_schedule_host",
     "gemm_variant_name",
     "one_shot_reduce",
     "signal_tiles",
@@ -297,6 +298,19 @@ def gemm_variant_name(dtype: torch.dtype, out_is_f32: bool, atomic: bool, varian
     buf = ctypes.create_string_buffer(128)
     err = _native.lib().iris_gemm_variant_name(_DTYPES[dtype], int(out_is_f32), int(atomic), variant, buf, 128)
     return None if err else buf.value.decode()
+
+
+def stream_k_schedule_host(total_tiles: int, k_steps: int, num_programs: int, pid: int):
+    """Items ``(tile, k_begin, k_end, parts)`` of program ``pid`` under the
+    kernels' stream-K schedule (host build of the same source)."""
+    cap = total_tiles + 2
+    items = (ctypes.c_int32 * (4 * cap))()
+    n = ctypes.c_int32()
+    err = _native.lib().iris_stream_k_schedule_host(total_tiles, k_steps, num_programs, pid, items, cap,
+                                                    ctypes.byref(n))
+    if err:
+        raise ValueError("iris_stream_k_schedule_host rejected the arguments")
+    return [tuple(items[4 * i:4 * i + 4]) for i in range(n.value)]
 
 
 def one_shot_reduce(c, c_global, tile_completed, heap_bases, rank, world_size, BLK_M, BLK_N, gsize_m, *,

@@ -108,3 +108,37 @@ def test_host_build_of_the_kernel_tile_map_is_bit_exact():
         want = O.tile_map_all(M, N, BM, BN, G)
         got = [ops.tile_map_host(t, M, N, BM, BN, G) for t in range(total)]
         assert got == [tuple(r) for r in want.tolist()]
+
+
+def test_host_build_of_the_stream_k_schedule_partitions_the_k_steps():
+    """The kernels' stream-K run arithmetic, compiled for the host: the runs
+    cut the launch's K-steps without gap or overlap, differ by at most one
+    step, every tile has exactly one owner, and the owner's count of parts is
+    the number of consecutive programs that hold the rest of its tile."""
+    from iris_amd import ops
+
+    for tiles, nk, programs in [(176, 64, 256), (24, 8, 5), (24, 8, 4), (5, 64, 8), (2, 128, 16), (20, 22, 24),
+                                (1024, 16, 256), (300, 16, 256), (1, 40, 7), (7, 3, 21)]:
+        sched = [ops.stream_k_schedule_host(tiles, nk, programs, pid) for pid in range(programs)]
+        lengths = [sum(ke - kb for _, kb, ke, _ in items) for items in sched]
+        assert sum(lengths) == tiles * nk and max(lengths) - min(lengths) <= 1
+        assert lengths == sorted(lengths, reverse=True)  # the longer runs come first
+        covered = {}
+        g = 0  # global step the next item must start at
+        for pid, items in enumerate(sched):
+            for n, (tile, kb, ke, parts) in enumerate(items):
+                assert 0 <= kb < ke <= nk and tile * nk + kb == g
+                assert kb == 0 or n == 0  # only a run's first item starts inside a tile
+                g = tile * nk + ke
+                for k in range(kb, ke):
+                    assert (tile, k) not in covered
+                    covered[(tile, k)] = pid
+                assert (parts == 0) == (kb != 0)
+        assert g == tiles * nk and len(covered) == tiles * nk
+        for pid, items in enumerate(sched):
+            for tile, kb, ke, parts in items:
+                if kb == 0:  # the owner: the rest of the tile is with the programs right after it
+                    holders = sorted({covered[(tile, k)] for k in range(nk)})
+                    assert holders == list(range(pid, pid + parts))
+    with pytest.raises(ValueError):
+        ops.stream_k_schedule_host(4, 4, 32, 0)  # runs would be empty
