@@ -50,6 +50,124 @@ int dbg() {
   return v;
 }
 
+// A few rows: the product is a stream over B, and the kernel built for that
+// takes it when the operands allow the 16-byte fetches, the logical tile
+// covers every row, the tiles' arrival counters have a home, and (with more
+// than 16 rows: two workgroups per 16 columns) every workgroup finds a place
+// on the device at once, so that B comes from HBM once.  Fills the plan and
+// returns true when the launch qualifies.
+bool plan_few_rows(const iris_gemm_args& a, int op, bool dma_ok, Plan* plan) {
+  GemmKArgs& k = plan->k;
+  const int64_t lim = (int64_t)1 << 31;
+  const int m_blocks = (a.M + SKINNY_ROWS - 1) / SKINNY_ROWS;
+  const int n_blocks = (a.N + SKINNY_COLS - 1) / SKINNY_COLS;
+  // fetches in flight per wave: enough for the whole K range, 8 blocks at most
+  const int per_wave = ((a.K + 63) / 64 + SKINNY_WAVES - 1) / SKINNY_WAVES;
+  const int un = per_wave <= 2 ? 2 : per_wave <= 4 ? 4 : 8;
+  const bool counters = (m_blocks == 1 && (a.block_n <= SKINNY_COLS || a.N <= SKINNY_COLS)) || k.flag_mode == 0 ||
+                        (a.locks && k.total_tiles <= a.num_sms);
+  bool room = true;
+  if (m_blocks > 1) {
+    int cus = 0, dev = 0;
+    const int per_cu = 160 * 1024 / skinny_lds_bytes(un) > 4 ? 4 : 160 * 1024 / skinny_lds_bytes(un);
+    room = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 &&
+           (int64_t)m_blocks * n_blocks <= (int64_t)cus * per_cu;
+  }
+  const bool ok = a.M <= SKINNY_MAX_ROWS && room && a.K > 0 && dma_ok && (op == OP_STORE16 || op == OP_STORE32) &&
+                  a.block_m >= a.M && (a.block_n % SKINNY_COLS) == 0 && !a.mm_begin_timestamp &&
+                  !a.mm_end_timestamp && (a.split_k == 0 || a.split_k == 1) && counters &&
+                  ((int64_t)SKINNY_ROWS * a.stride_am + a.K) * 2 < lim &&
+                  ((int64_t)SKINNY_COLS * a.stride_bn + a.K) * 2 < lim;
+  if (!ok) return false;
+  plan->skinny = gemm_skinny_kernel_for(a.ab_dtype, op, un);
+  if (!plan->skinny) return false;
+  plan->skinny_lds = skinny_lds_bytes(un);
+  plan->skinny_grid = n_blocks;
+  plan->skinny_grid_y = m_blocks;
+  k.split_k = 1;
+  k.locks = a.locks;
+  return true;
+}
+
+// Split-K and stream-K.  The owner of a tile waits for the programs that hold
+// its other parts, so every part needs a program of its own that is resident
+// at the same time: no more programs than the device has CUs.
+hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, GemmKArgs* kp) {
+  GemmKArgs& k = *kp;
+  k.split_k = 1;
+  k.split_q = k.split_r = 0;
+  k.partials = a.partials;
+  k.locks = a.locks;
+  k.partial_stride = a.partials_slot_elems;
+  k.status = a.status;
+  k.timeout = a.spin_timeout_ticks ? a.spin_timeout_ticks : 200000000ull;  // 2 s at 100 MHz
+  k.stream_k = 0;
+  if (a.split_k < 0 && a.split_k != IRIS_GEMM_SPLIT_STREAM_K) return hipErrorInvalidValue;
+  const int nk = (a.K + pick.bk - 1) / pick.bk;
+  if (a.split_k != 1 && a.partials && a.locks) {
+    int cus = 0, dev = 0;
+    const bool resident = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 && a.num_sms <= cus;
+    const bool possible = resident && pick.splitk && pick.fn_split && k.sub_m == 1 && k.sub_n == 1 &&
+                          a.partials_slot_elems >= (int64_t)pick.cm * pick.cn &&
+                          (reinterpret_cast<uintptr_t>(a.partials) & 15) == 0 && (a.partials_slot_elems % 4) == 0;
+    // Stream-K: every program takes the same number of K-steps (within one).
+    // A run of at least four steps keeps the parts of a tile few.
+    const int64_t steps = (int64_t)k.total_tiles * nk;
+    const int run = (int)(steps / a.num_sms);
+    const bool stream_ok = possible && run >= 4 && steps < ((int64_t)1 << 30) && (nk + run - 1) / run + 1 <= 32;
+    if (a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
+      if (!stream_ok) return hipErrorInvalidValue;
+      k.stream_k = 1;
+    } else if (a.split_k > 1) {
+      if (!possible || a.split_k > nk || a.split_k > 64 || (int64_t)k.total_tiles * a.split_k > a.num_sms)
+        return hipErrorInvalidValue;
+      k.split_k = a.split_k;
+    } else if (possible) {
+      // K-steps a program walks through, unsplit
+      const int rounds = (k.total_tiles + a.num_sms - 1) / a.num_sms;
+      int walk = rounds * nk;
+      if (k.total_tiles * 2 <= a.num_sms && nk >= 32) {
+        // The hand-over of partials costs about as much as ten K-steps of a
+        // small tile, so only long K loops are split: as many parts as there
+        // are idle programs, at least four K-steps each.
+        int sk = a.num_sms / k.total_tiles;
+        if (sk > nk / 4) sk = nk / 4;
+        if (sk > 16) sk = 16;
+        if (sk > 1) {
+          k.split_k = sk;
+          walk = (nk + sk - 1) / sk;
+        }
+      }
+      // Stream-K when it shortens that walk by 15 % or more.  With runs of at
+      // least a tile's length a tile spans two runs and the second hands its
+      // part over first thing, long before the owner asks: nothing is lost.
+      // With shorter runs the owner waits for programs that finish when it
+      // does, and more CUs pull operands at once; measured on the decoder
+      // shapes that pays when the walk is long and at least 45 % shorter than
+      // the unsplit one (132 tiles of 64 steps on 256 programs: -17 %; 176
+      // tiles: +9 %; 22-step tiles: +6 to +20 %).
+      const bool hidden = run >= nk;
+      if (stream_ok && nk >= 16 && run >= 8 && (int64_t)(run + 1) * 20 <= (int64_t)walk * 17 &&
+          (hidden || (nk >= 32 && (int64_t)(run + 1) * 20 <= (int64_t)rounds * nk * 11))) {
+        k.stream_k = 1;
+        k.split_k = 1;
+      }
+    }
+  } else if (a.split_k > 1 || a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
+    return hipErrorInvalidValue;  // forced, but no workspace
+  }
+  if (k.split_k > 1) {
+    k.split_q = nk / k.split_k;
+    k.split_r = nk % k.split_k;
+  }
+  if (k.stream_k) {
+    const int64_t steps = (int64_t)k.total_tiles * nk;
+    k.split_q = (int)(steps / a.num_sms);
+    k.split_r = (int)(steps % a.num_sms);
+  }
+  return hipSuccess;
+}
+
 // Validate `a` and build the launch plan.  Returns hipSuccess,
 // hipErrorInvalidValue, or a pseudo-success with entry == nullptr when there
 // is no GEMM work to do.
@@ -152,41 +270,8 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
     return ((int64_t)e.cm * a.stride_am + a.K) * 2 < lim && ((int64_t)e.cn * a.stride_bn + a.K) * 2 < lim;
   };
 
-  // A few rows: the product is a stream over B, and the kernel built for
-  // that takes it when the operands allow the 16-byte fetches, the logical
-  // tile covers every row, the tiles' arrival counters have a home, and (with
-  // more than 16 rows: two workgroups per 16 columns) every workgroup finds
-  // a place on the device at once, so that B comes from HBM once.
   if (a.variant == 0 || a.variant == IRIS_GEMM_VARIANT_FEW_ROWS) {
-    const int64_t lim = (int64_t)1 << 31;
-    const int m_blocks = (a.M + SKINNY_ROWS - 1) / SKINNY_ROWS;
-    const int n_blocks = (a.N + SKINNY_COLS - 1) / SKINNY_COLS;
-    const int per_wave = ((a.K + 63) / 64 + SKINNY_WAVES - 1) / SKINNY_WAVES;
-    const int un = per_wave <= 2 ? 2 : per_wave <= 4 ? 4 : 8;
-    const bool counters = (m_blocks == 1 && (a.block_n <= SKINNY_COLS || a.N <= SKINNY_COLS)) || k.flag_mode == 0 ||
-                          (a.locks && k.total_tiles <= a.num_sms);
-    bool room = true;
-    if (m_blocks > 1) {
-      int cus = 0, dev = 0;
-      const int per_cu = 160 * 1024 / skinny_lds_bytes(un) > 4 ? 4 : 160 * 1024 / skinny_lds_bytes(un);
-      room = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 &&
-             (int64_t)m_blocks * n_blocks <= (int64_t)cus * per_cu;
-    }
-    const bool ok = a.M <= SKINNY_MAX_ROWS && room && a.K > 0 && dma_ok && (op == OP_STORE16 || op == OP_STORE32) &&
-                    a.block_m >= a.M && (a.block_n % SKINNY_COLS) == 0 && !a.mm_begin_timestamp &&
-                    !a.mm_end_timestamp && (a.split_k == 0 || a.split_k == 1) && counters &&
-                    ((int64_t)SKINNY_ROWS * a.stride_am + a.K) * 2 < lim &&
-                    ((int64_t)SKINNY_COLS * a.stride_bn + a.K) * 2 < lim;
-    if (ok) {
-      // (un: fetches in flight per wave, enough for the whole K range, 8 blocks at most)
-      plan->skinny = gemm_skinny_kernel_for(a.ab_dtype, op, un);
-      plan->skinny_lds = skinny_lds_bytes(un);
-      plan->skinny_grid = n_blocks;
-      plan->skinny_grid_y = m_blocks;
-      k.split_k = 1;
-      k.locks = a.locks;
-      if (plan->skinny) return hipSuccess;
-    }
+    if (plan_few_rows(a, op, dma_ok, plan)) return hipSuccess;
     if (a.variant == IRIS_GEMM_VARIANT_FEW_ROWS) return hipErrorInvalidValue;
   }
 
@@ -227,82 +312,9 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   k.sub_n = (span_n + pick->cn - 1) / pick->cn;
   plan->entry = pick;
 
-  // Split-K.  The owner of a tile waits for the programs that hold its other
-  // parts, so every (tile, part) pair needs a program of its own that is
-  // resident at the same time: one pair per program, and no more programs
-  // than the device has CUs.
-  k.split_k = 1;
-  k.split_q = k.split_r = 0;
-  k.partials = a.partials;
-  k.locks = a.locks;
-  k.partial_stride = a.partials_slot_elems;
-  k.status = a.status;
-  k.timeout = a.spin_timeout_ticks ? a.spin_timeout_ticks : 200000000ull;  // 2 s at 100 MHz
-  k.stream_k = 0;
-  if (a.split_k < 0 && a.split_k != IRIS_GEMM_SPLIT_STREAM_K) return hipErrorInvalidValue;
-  const int nk = (a.K + pick->bk - 1) / pick->bk;
-  if (a.split_k != 1 && a.partials && a.locks) {
-    int cus = 0, dev = 0;
-    const bool resident = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 && a.num_sms <= cus;
-    const bool possible = resident && pick->splitk && pick->fn_split && k.sub_m == 1 && k.sub_n == 1 &&
-                          a.partials_slot_elems >= (int64_t)pick->cm * pick->cn &&
-                          (reinterpret_cast<uintptr_t>(a.partials) & 15) == 0 && (a.partials_slot_elems % 4) == 0;
-    // Stream-K: every program takes the same number of K-steps (within one).
-    // A run of at least four steps keeps the parts of a tile few.
-    const int64_t steps = (int64_t)k.total_tiles * nk;
-    const int run = (int)(steps / a.num_sms);
-    const bool stream_ok = possible && run >= 4 && steps < ((int64_t)1 << 30) && (nk + run - 1) / run + 1 <= 32;
-    if (a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
-      if (!stream_ok) return hipErrorInvalidValue;
-      k.stream_k = 1;
-    } else if (a.split_k > 1) {
-      if (!possible || a.split_k > nk || a.split_k > 64 || (int64_t)k.total_tiles * a.split_k > a.num_sms)
-        return hipErrorInvalidValue;
-      k.split_k = a.split_k;
-    } else if (possible) {
-      // K-steps a program walks through, unsplit
-      const int rounds = (k.total_tiles + a.num_sms - 1) / a.num_sms;
-      int walk = rounds * nk;
-      if (k.total_tiles * 2 <= a.num_sms && nk >= 32) {
-        // The hand-over of partials costs about as much as ten K-steps of a
-        // small tile, so only long K loops are split: as many parts as there
-        // are idle programs, at least four K-steps each.
-        int sk = a.num_sms / k.total_tiles;
-        if (sk > nk / 4) sk = nk / 4;
-        if (sk > 16) sk = 16;
-        if (sk > 1) {
-          k.split_k = sk;
-          walk = (nk + sk - 1) / sk;
-        }
-      }
-      // Stream-K when it shortens that walk by 15 % or more.  With runs of at
-      // least a tile's length a tile spans two runs and the second hands its
-      // part over first thing, long before the owner asks: nothing is lost.
-      // With shorter runs the owner waits for programs that finish when it
-      // does, and more CUs pull operands at once; measured on the decoder
-      // shapes that pays when the walk is long and at least 45 % shorter than
-      // the unsplit one (132 tiles of 64 steps on 256 programs: -17 %; 176
-      // tiles: +9 %; 22-step tiles: +6 to +20 %).
-      const bool hidden = run >= nk;
-      if (stream_ok && nk >= 16 && run >= 8 && (int64_t)(run + 1) * 20 <= (int64_t)walk * 17 &&
-          (hidden || (nk >= 32 && (int64_t)(run + 1) * 20 <= (int64_t)rounds * nk * 11))) {
-        k.stream_k = 1;
-        k.split_k = 1;
-      }
-    }
-  } else if (a.split_k > 1 || a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
-    return hipErrorInvalidValue;  // forced, but no workspace
-  }
-  if (k.split_k > 1) {
-    k.split_q = nk / k.split_k;
-    k.split_r = nk % k.split_k;
-  }
-  if (k.stream_k) {
-    const int64_t steps = (int64_t)k.total_tiles * nk;
-    k.split_q = (int)(steps / a.num_sms);
-    k.split_r = (int)(steps % a.num_sms);
-    return hipSuccess;  // (every program has a run: the reference's XCD remap stays)
-  }
+  const hipError_t err = plan_split(a, *pick, &k);
+  // (under stream-K every program has a run: the reference's XCD remap stays)
+  if (err != hipSuccess || k.stream_k) return err;
   // Fewer (tile, part) items than programs: deal them to the XCDs evenly, in
   // consecutive runs, instead of filling the first XCDs and idling the rest.
   const int64_t work = (int64_t)k.total_tiles * k.split_k;
