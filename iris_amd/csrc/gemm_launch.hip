@@ -2,6 +2,8 @@
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
+#include <utility>
+#include <vector>
 
 #include "gemm_skinny.hpp"
 
@@ -323,11 +325,18 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
 }
 
 hipError_t ensure_lds(GemmKernelFn fn, int lds_bytes) {
-  // dynamic LDS above 64 KiB must be opted into once per function
+  // dynamic LDS above 64 KiB must be opted into once per function and device
   static std::mutex m;
+  static std::vector<std::pair<int, GemmKernelFn>> done;
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
   std::lock_guard<std::mutex> lock(m);
-  return hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                             lds_bytes);
+  for (const auto& d : done)
+    if (d.first == dev && d.second == fn) return hipSuccess;
+  err = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  if (err == hipSuccess) done.emplace_back(dev, fn);
+  return err;
 }
 
 iris_reduce_args reduce_args_from(const iris_gemm_args& a) {
