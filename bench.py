@@ -61,6 +61,8 @@ def parse():
                     help="headline: the 8192x8192x1024 shard GEMM + reduce (the metric's configuration); atomic: eight "
                          "K-shard GEMMs adding into one fp32 C; decoder: 6.7B-decoder-shaped shards for M in "
                          "{1,16,128,512,2048}.  The last two print their own JSON line.")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="headline run: skip the atomic-accumulate and decoder-shard summaries")
     ap.add_argument("--no-context", action="store_true",
                     help="skip the two context figures: the library GEMM and the matrix cores' sustained rate")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -211,7 +213,7 @@ def context_figures(a, b, c_global, flops):
     return out
 
 
-def run_atomic(args):
+def run_atomic(args, emit=True):
     """BASELINE config 4: eight sequential bf16 K-shard GEMMs A_i[4096,512] x
     B_i[512,4096], each adding its tiles with fp32 atomics into one C[4096,4096]
     in the heap."""
@@ -248,7 +250,7 @@ def run_atomic(args):
     ms = steady_ms(step, n=max(10, args.steps // 10))
     flops = 2.0 * Ma * Na * ks * shards
     updates = Ma * Na * shards
-    print(json.dumps({
+    result = {
         "metric": "atomic-accumulate epilogue: 8 K-shard GEMMs into one fp32 C", "value": round(flops / ms / 1e9, 2),
         "unit": "TFLOP/s", "n_gpus": 1, "ms_per_step": round(ms, 5), "higher_is_better": True, "dtype": "bf16",
         "data": "synthetic",
@@ -257,10 +259,13 @@ def run_atomic(args):
         "atomic_updates_per_s": round(updates / (ms * 1e-3), 0),
         "atomic_GBps_at_4B": round(updates * 4 / (ms * 1e-3) / 1e9, 1),
         "max_abs_err_vs_fp32": err,
-    }))
+    }
+    if emit:
+        print(json.dumps(result))
+    return result
 
 
-def run_decoder(args):
+def run_decoder(args, emit=True):
     """BASELINE config 5: 6.7B-decoder-shaped shards (hidden 4096, FFN 11008,
     1/8 shard = 1376).  Gate/up: [M,4096] x [4096,1376] scattered into every
     rank's [M, 8*1376] at column rank*1376; down: [M,1376] x [1376,4096] as a
@@ -364,13 +369,16 @@ def run_decoder(args):
         })
         shmem.heap_offset = off  # the next M reuses the heap
     big = rows[-1]
-    print(json.dumps({
+    result = {
         "metric": "decoder-shaped shard GEMMs (hidden 4096, FFN 11008 / 8)", "value": big["gate_up_tflops"],
         "unit": "TFLOP/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "gate/up [M,4096]x[4096,1376] all-scatter to 8 ranks + down [M,1376]x[1376,4096] "
                                "fp32 partial + one-shot reduce of 8 partials; value = gate/up at M=2048"},
         "per_M": rows,
-    }))
+    }
+    if emit:
+        print(json.dumps(result))
+    return result
 
 
 def main():
@@ -538,6 +546,17 @@ def main():
         assert torch.equal(src, dst)
         result["copy_calibration"] = {"kernel": "reduce_tiles_vec_kernel<fp32, fp32, ws=1>",
                                       "read_bytes": M * N * 4, "write_bytes": M * N * 4, "launches": 3}
+
+    if not args.no_context and not args.no_other_workloads:
+        # the other configurations, each measured as its own --workload run measures it
+        at = run_atomic(args, emit=False)
+        dec = run_decoder(args, emit=False)
+        keep = ("M", "kernel_up", "split_k_up", "gate_up_us", "gate_up_tflops", "gate_up_weight_GBps", "kernel_down",
+                "split_k_down", "down_us", "down_tflops", "reduce_us", "reduce_GBps")
+        result["other_workloads"] = {
+            "atomic_accumulate": {k: at[k] for k in ("value", "unit", "ms_per_step", "atomic_updates_per_s", "config")},
+            "decoder_shards": {"config": dec["config"], "per_M": [{k: r[k] for k in keep} for r in dec["per_M"]]},
+        }
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
