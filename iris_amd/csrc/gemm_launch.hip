@@ -75,7 +75,7 @@ bool plan_few_rows(const iris_gemm_args& a, int op, bool dma_ok, Plan* plan) {
     room = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 &&
            (int64_t)m_blocks * n_blocks <= (int64_t)cus * per_cu;
   }
-  const bool ok = a.M <= SKINNY_MAX_ROWS && room && a.K > 0 && dma_ok && (op == OP_STORE16 || op == OP_STORE32) &&
+  const bool ok = a.M <= SKINNY_MAX_ROWS && room && a.K > 0 && dma_ok &&
                   a.block_m >= a.M && (a.block_n % SKINNY_COLS) == 0 && !a.mm_begin_timestamp &&
                   !a.mm_end_timestamp && (a.split_k == 0 || a.split_k == 1) && counters &&
                   ((int64_t)SKINNY_ROWS * a.stride_am + a.K) * 2 < lim &&

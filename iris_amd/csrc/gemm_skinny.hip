@@ -7,7 +7,7 @@ namespace {
 
 template <int DT, int OP>
 GemmKernelFn pick_un(int un) {
-  constexpr int ODT = OP == OP_STORE32 ? IRIS_DTYPE_F32 : DT;
+  constexpr int ODT = (OP == OP_STORE32 || OP == OP_ATOMIC32) ? IRIS_DTYPE_F32 : DT;
   switch (un) {
     case 2: return &gemm_skinny_kernel<DT, OP, ODT, 2>;
     case 4: return &gemm_skinny_kernel<DT, OP, ODT, 4>;
@@ -22,9 +22,13 @@ GemmKernelFn gemm_skinny_kernel_for(int dt, int op, int un) {
   if (dt == IRIS_DTYPE_BF16) {
     if (op == OP_STORE16) return pick_un<IRIS_DTYPE_BF16, OP_STORE16>(un);
     if (op == OP_STORE32) return pick_un<IRIS_DTYPE_BF16, OP_STORE32>(un);
+    if (op == OP_ATOMIC32) return pick_un<IRIS_DTYPE_BF16, OP_ATOMIC32>(un);
+    if (op == OP_ATOMIC16) return pick_un<IRIS_DTYPE_BF16, OP_ATOMIC16>(un);
   } else if (dt == IRIS_DTYPE_F16) {
     if (op == OP_STORE16) return pick_un<IRIS_DTYPE_F16, OP_STORE16>(un);
     if (op == OP_STORE32) return pick_un<IRIS_DTYPE_F16, OP_STORE32>(un);
+    if (op == OP_ATOMIC32) return pick_un<IRIS_DTYPE_F16, OP_ATOMIC32>(un);
+    if (op == OP_ATOMIC16) return pick_un<IRIS_DTYPE_F16, OP_ATOMIC16>(un);
   }
   return nullptr;
 }

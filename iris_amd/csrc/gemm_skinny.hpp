@@ -1,6 +1,6 @@
 // Shard GEMM for a few rows of A (decode-time batches, 16 rows a workgroup): C[M,N] = A[M,K] B[K,N]
-// with the store epilogues of the persistent kernel (gemm_all_scatter.py:209-251,
-// gemm_one_shot_all_reduce.py:197-218).
+// with the epilogues of the persistent kernel (gemm_all_scatter.py:209-251,
+// gemm_atomics_all_reduce.py:236-248, gemm_one_shot_all_reduce.py:197-218).
 //
 // With so few rows the product is a stream over B: every byte of B is used
 // once, the matrix cores idle, and what matters is how many bytes a CU has in
@@ -40,7 +40,8 @@ constexpr int skinny_lds_bytes(int un) { return SKINNY_RED_BYTES + SKINNY_WAVES 
 template <int DT, int OP, int ODT, int UN>
 __global__ __launch_bounds__(SKINNY_THREADS) __attribute__((amdgpu_waves_per_eu(2, UN == 8 ? 2 : UN == 4 ? 4 : 8))) void
 gemm_skinny_kernel(const GemmKArgs p) {
-  static_assert(OP == OP_STORE16 || OP == OP_STORE32, "store epilogues only");
+  constexpr bool ATOMIC = OP == OP_ATOMIC32 || OP == OP_ATOMIC16;
+  constexpr bool F32 = OP == OP_STORE32 || OP == OP_ATOMIC32;
   using vec8 = typename Mfma<DT>::vec8;
   extern __shared__ __attribute__((aligned(1024))) char skinny_lds[];
   IRIS_LDS char* lds = (IRIS_LDS char*)skinny_lds;
@@ -124,13 +125,29 @@ gemm_skinny_kernel(const GemmKArgs p) {
     f32x4 s = red[lane];
 #pragma unroll
     for (int w = 1; w < SKINNY_WAVES; ++w) s += red[w * 64 + lane];  // wave order: the sum does not depend on timing
-    constexpr int ES = OP == OP_STORE32 ? 4 : 2;
+    constexpr int ES = F32 ? 4 : 2;
     const bool whole = p.vec_out && n + 4 <= p.N;
     for (int r = r_begin + wave; r < r_end; r += SKINNY_WAVES) {
       IRIS_GLOBAL char* dst = rank_ptr(p, p.out, r);
-      if (whole) {
+      if constexpr (ATOMIC) {
+        // 08: add into the destination (gemm_atomics_all_reduce.py:236-248)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (n + e >= p.N) continue;
+          IRIS_GLOBAL char* d = dst + ((int64_t)m * p.som + (int64_t)(n + e) * p.son) * ES;
+          const float f = s[e];
+          if constexpr (OP == OP_ATOMIC32) {
+            __hip_atomic_fetch_add((IRIS_GLOBAL float*)d, f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          } else if (whole && (e & 1) == 0) {
+            atomic_add16_pair<ODT>((IRIS_GLOBAL unsigned int*)d, pack2<ODT>(s[e], s[e + 1]));
+            ++e;  // the pair took the next column too
+          } else {
+            atomic_add16_cas<ODT>((IRIS_GLOBAL unsigned short*)d, from16<ODT>(to16<ODT>(f)));
+          }
+        }
+      } else if (whole) {
         IRIS_GLOBAL unsigned int* d = (IRIS_GLOBAL unsigned int*)(dst + ((int64_t)m * p.som + n) * ES);
-        if constexpr (OP == OP_STORE32) {
+        if constexpr (F32) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const float f = s[e];  // (a bit cast of the element itself reads element 0)
@@ -146,7 +163,7 @@ gemm_skinny_kernel(const GemmKArgs p) {
           if (n + e >= p.N) continue;
           IRIS_GLOBAL char* d = dst + ((int64_t)m * p.som + (int64_t)(n + e) * p.son) * ES;
           const float f = s[e];
-          if constexpr (OP == OP_STORE32)
+          if constexpr (F32)
             store_through((IRIS_GLOBAL unsigned int*)d, __builtin_bit_cast(unsigned int, f), p.sys != 0);
           else
             store_through((IRIS_GLOBAL unsigned short*)d, to16<ODT>(s[e]), p.sys != 0);

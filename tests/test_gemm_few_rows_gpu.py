@@ -176,6 +176,34 @@ def test_one_shot_fused_phase(shmem, ws):
     assert not shmem.on_rank(flags, last).any()  # consumed
 
 
+@pytest.mark.parametrize("M,out_dtype", [(16, torch.float32), (24, torch.float32), (7, torch.bfloat16),
+                                         (32, torch.bfloat16)])
+def test_atomic_accumulate_of_k_shards(shmem, M, out_dtype):
+    """08 epilogue: every rank adds its K-shard product into every rank's C."""
+    ws, N, K, BM, BN, dtype = 4, 208, 4 * 320, 32, 64, torch.bfloat16
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    shards = O.k_shards(A, B, ws)
+    ah, bh = to_heap(shmem, A), to_heap(shmem, B)
+    kk = K // ws
+    c = shmem.zeros((M, N), dtype=out_dtype)
+    hb = shmem.get_heap_bases()
+    for r in range(ws):
+        shmem.on_rank(c, r).zero_()
+    for r in range(ws):
+        args = (ah[:, r * kk:(r + 1) * kk], bh[r * kk:(r + 1) * kk, :], None, shmem.on_rank(c, r), None, hb, r, ws, 256,
+                BM, BN, 64, 4, ops.EPI_ATOMIC_ADD)
+        assert ops.gemm_plan_name(*args) == FEW
+        ops.gemm_launch(*args)
+    torch.cuda.synchronize()
+    want = O.atomics_all_reduce(shards)
+    for r in range(ws):
+        got = shmem.on_rank(c, r).float().cpu()
+        if out_dtype == torch.float32:
+            check_close(got, want, f"rank {r}")
+        else:  # 16-bit accumulation rounds after every add: 4 roundings of half an ulp each
+            assert float((got - want).abs().max()) <= 4 * 2.0 ** -8 * float(want.abs().max()) + 1e-2, f"rank {r}"
+
+
 def test_choice_of_kernel(shmem):
     dtype = torch.bfloat16
     A, B = make_ab(16, 256, 128, dtype)
@@ -213,9 +241,8 @@ def test_choice_of_kernel(shmem):
     # B with N contiguous: no 16-byte fetches along K
     bn = shmem.zeros((128, 256), dtype=dtype)
     assert plan(a, bn, cg, 64, 64, locks=locks) != FEW
-    # atomics keep the persistent kernel
-    assert ops.gemm_plan_name(a, b, None, cg, flags, hb, 0, 1, 256, 64, 64, 64, 4, ops.EPI_ATOMIC_ADD,
-                              locks=locks) != FEW
+    # the atomic epilogue publishes nothing: no counters needed
+    assert ops.gemm_plan_name(a, b, None, cg, flags, hb, 0, 1, 256, 64, 64, 64, 4, ops.EPI_ATOMIC_ADD) == FEW
 
 
 def test_persistent_choice_gives_the_same_result(shmem):
