@@ -173,6 +173,32 @@ typedef struct iris_gemm_args {
  */
 int iris_gemm_launch(const iris_gemm_args* args, void* stream);
 
+/*
+ * iris_gemm_launch for callers that cannot allocate device memory and have no
+ * workspace to pass: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference
+ * (whose wrappers allocate `P` and `locks` with torch, benchmark.py:136-142).
+ * `args->partials`, `args->locks` and `args->partials_slot_elems` are ignored:
+ * the split-K / stream-K partial tiles and the locks (also the few-rows
+ * kernel's arrival counters) live in a device array inside the library,
+ * IRIS_GEMM_NOALLOC_MAX_PROGRAMS slots of IRIS_GEMM_NOALLOC_MAX_TILE_ELEMS
+ * floats plus 4 KiB of locks (16 MiB + 4 KiB per device, held until the process
+ * ends).  The call allocates and frees nothing; it clears the locks with a
+ * fill kernel on `stream` before the GEMM when the launch uses them.
+ * Limits: num_sms > IRIS_GEMM_NOALLOC_MAX_PROGRAMS is rejected; a forced split
+ * (split_k > 1 or IRIS_GEMM_SPLIT_STREAM_K) with block_m * block_n >
+ * IRIS_GEMM_NOALLOC_MAX_TILE_ELEMS is rejected; both print the reason to
+ * stderr and return hipErrorInvalidValue.  With split_k == 0 a larger tile
+ * runs unsplit, as iris_gemm_launch does without a workspace.
+ * Every call on a device shares that device's array: calls that overlap on
+ * one device (two streams, two threads) race on it.  The first call on a
+ * device looks the array's address up (hipGetSymbolAddress) and should be made
+ * outside a graph capture.
+ */
+#define IRIS_GEMM_NOALLOC_MAX_PROGRAMS 256
+#define IRIS_GEMM_NOALLOC_MAX_TILE_ELEMS 16384 /* 128 x 128, the largest tile with a split-K build */
+int iris_gemm_launch_noalloc(const iris_gemm_args* args, void* stream);
+
 /* Registers and spills of the kernel `iris_gemm_launch` would pick for `args`
  * (what the reference reads from kk.n_regs / kk.n_spills,
  * matmul_wrapper.py:152-155).  *spills is the scratch bytes per lane. */

@@ -131,6 +131,7 @@ SIGNATURES = {
     "iris_hip_device_synchronize": (_I, []),
     "iris_hip_arch_name": (_I, [_I, ctypes.c_char_p, ctypes.c_size_t]),
     "iris_gemm_launch": (_I, [ctypes.POINTER(GemmArgs), _P]),
+    "iris_gemm_launch_noalloc": (_I, [ctypes.POINTER(GemmArgs), _P]),
     "iris_gemm_kernel_info": (_I, [ctypes.POINTER(GemmArgs), ctypes.POINTER(_I), ctypes.POINTER(_I)]),
     "iris_gemm_split_k": (_I, [ctypes.POINTER(GemmArgs), ctypes.POINTER(_I)]),
     "iris_gemm_variant_name": (_I, [_I, _I, _I, _I, ctypes.c_char_p, ctypes.c_size_t]),

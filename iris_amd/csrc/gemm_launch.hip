@@ -373,11 +373,11 @@ iris_reduce_args reduce_args_from(const iris_gemm_args& a) {
 
 using namespace iris_amd;
 
-extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
-  if (!args) return hipErrorInvalidValue;
-  Plan plan;
-  hipError_t err = make_plan(*args, &plan);
-  if (err != hipSuccess) return err;
+namespace {
+
+// Enqueue what `plan` describes on `stream`.
+hipError_t run_plan(const Plan& plan, const iris_gemm_args& args, void* stream) {
+  hipError_t err = hipSuccess;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (plan.skinny) {
     if (dbg())
@@ -410,10 +410,109 @@ extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
     // the same stream: it waits for each tile's flag, sums the partials and
     // stores the result, exactly what the tail of the reference program does
     // for that tile (gemm_one_shot_all_reduce.py:220-271).
-    const iris_reduce_args r = reduce_args_from(*args);
-    return iris_one_shot_reduce_launch(&r, stream);
+    const iris_reduce_args r = reduce_args_from(args);
+    return static_cast<hipError_t>(iris_one_shot_reduce_launch(&r, stream));
   }
   return hipSuccess;
+}
+
+}  // namespace
+
+extern "C" int iris_gemm_launch(const iris_gemm_args* args, void* stream) {
+  if (!args) return hipErrorInvalidValue;
+  Plan plan;
+  hipError_t err = make_plan(*args, &plan);
+  if (err != hipSuccess) return err;
+  return run_plan(plan, *args, stream);
+}
+
+// ---------------------------------------------------------------------------
+// The launch that allocates nothing: the split-K / stream-K / few-rows
+// workspace (partial tiles and their locks) lives in a device array of this
+// library instead of in buffers of the caller.
+// ---------------------------------------------------------------------------
+
+namespace {
+
+constexpr size_t NOALLOC_LOCK_BYTES = 4096;  // int32[1024]: one lock per program or tile
+constexpr size_t NOALLOC_PARTIAL_BYTES =
+    (size_t)IRIS_GEMM_NOALLOC_MAX_PROGRAMS * IRIS_GEMM_NOALLOC_MAX_TILE_ELEMS * sizeof(float);
+constexpr size_t NOALLOC_BYTES = NOALLOC_LOCK_BYTES + NOALLOC_PARTIAL_BYTES;
+
+}  // namespace
+
+// locks first, then one partial-tile slot per program.  Every device the
+// library runs on holds its own copy until the process ends.
+static __device__ __align__(256) unsigned char scratch[NOALLOC_BYTES];
+
+namespace {
+
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* p, int32_t v, int n) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) p[i] = v;
+}
+
+// Device address of `scratch` on the current device, looked up once per
+// device.  (In host code the array's name is only a handle for this lookup.)
+hipError_t scratch_address(unsigned char** out) {
+  static std::mutex m;
+  static unsigned char* ptr[64] = {};
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(m);
+  if (!ptr[dev]) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return err;
+    if (!p) return hipErrorInvalidSymbol;
+    ptr[dev] = static_cast<unsigned char*>(p);
+  }
+  *out = ptr[dev];
+  return hipSuccess;
+}
+
+}  // namespace
+
+extern "C" int iris_gemm_launch_noalloc(const iris_gemm_args* args, void* stream) {
+  if (!args) return hipErrorInvalidValue;
+  if (args->num_sms > IRIS_GEMM_NOALLOC_MAX_PROGRAMS) {
+    std::fprintf(stderr, "[iris_amd] iris_gemm_launch_noalloc: num_sms %d exceeds the workspace's %d programs\n",
+                 args->num_sms, IRIS_GEMM_NOALLOC_MAX_PROGRAMS);
+    return hipErrorInvalidValue;
+  }
+  const int64_t tile_elems = (int64_t)args->block_m * args->block_n;
+  const bool forced = args->split_k > 1 || args->split_k == IRIS_GEMM_SPLIT_STREAM_K;
+  if (forced && tile_elems > IRIS_GEMM_NOALLOC_MAX_TILE_ELEMS) {
+    std::fprintf(stderr,
+                 "[iris_amd] iris_gemm_launch_noalloc: a split of K was asked for, and a %d x %d tile exceeds the "
+                 "workspace's %d elements per partial tile\n",
+                 args->block_m, args->block_n, IRIS_GEMM_NOALLOC_MAX_TILE_ELEMS);
+    return hipErrorInvalidValue;
+  }
+  unsigned char* base = nullptr;
+  hipError_t err = scratch_address(&base);
+  if (err != hipSuccess) return err;
+
+  iris_gemm_args a = *args;
+  a.locks = reinterpret_cast<int32_t*>(base);
+  // tiles beyond the slot size run unsplit, exactly as without a workspace
+  a.partials = tile_elems <= IRIS_GEMM_NOALLOC_MAX_TILE_ELEMS ? reinterpret_cast<float*>(base + NOALLOC_LOCK_BYTES) : nullptr;
+  a.partials_slot_elems = a.partials ? IRIS_GEMM_NOALLOC_MAX_TILE_ELEMS : 0;
+  Plan plan;
+  err = make_plan(a, &plan);
+  if (err != hipSuccess) return err;
+  // The array keeps what the last call left: the locks must start at zero (a
+  // wait that timed out leaves one raised).  A fill kernel, not a memset, so
+  // that the call can be recorded into a HIP graph.
+  const bool uses_locks = (plan.skinny && plan.k.flag_mode != 0) || (plan.entry && (plan.k.split_k > 1 || plan.k.stream_k));
+  if (uses_locks) {
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), a.locks, 0,
+                       (int)(NOALLOC_LOCK_BYTES / sizeof(int32_t)));
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+  }
+  return run_plan(plan, a, stream);
 }
 
 extern "C" int iris_gemm_split_k(const iris_gemm_args* args, int* split_k) {

@@ -59,6 +59,6 @@ int iris_hip_arch_name(int device, char* buf, size_t len) {
   return hipSuccess;
 }
 
-int iris_amd_abi_version(void) { return 3; }
+int iris_amd_abi_version(void) { return 4; }
 
 }  // extern "C"

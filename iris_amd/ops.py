@@ -55,6 +55,9 @@ __all__ = [
 
 _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
 
+# limits of iris_gemm_launch_noalloc (include/iris_amd.h)
+NOALLOC_MAX_PROGRAMS, NOALLOC_MAX_TILE_ELEMS = 256, 16384
+
 # iris_rma_selftest_launch (include/iris_amd.h)
 RMA_OPS = {"load": 0, "store": 1, "get": 2, "put": 3, "atomic_add": 4, "atomic_sub": 5, "atomic_cas": 6,
            "atomic_xchg": 7}
@@ -224,7 +227,7 @@ def _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_s
 def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
                 gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, scope=SCOPE_AGENT, variant=0,
                 mm_begin_timestamp=None, mm_end_timestamp=None, status=None, spin_timeout_ticks=0, partials=None,
-                locks=None, split_k=0):
+                locks=None, split_k=0, noalloc=False):
     """Launch the persistent shard GEMM ``a @ b`` with a tile-publishing epilogue.
 
     ``partials`` / ``locks`` are the wrappers' ``P`` and ``locks`` buffers
@@ -234,14 +237,33 @@ def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size,
     runs of K-steps (stream-K, ``split_k=SPLIT_STREAM_K`` to insist) (``split_k`` 0:
     the launcher decides, 1: never, n: exactly n).
 
+    ``noalloc=True`` goes through ``iris_gemm_launch_noalloc``: no workspace
+    is passed, the library's own device array takes its place.
+
     The kernel launch of the reference wrappers (matmul_wrapper.py:109-150).
     """
-    args = _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N,
-                           BLK_K, gsize_m, epilogue, phase, notify, num_xcds, scope, variant, mm_begin_timestamp,
-                           mm_end_timestamp, status, spin_timeout_ticks, partials, locks, split_k)
+    if noalloc:
+        if partials is not None or locks is not None:
+            raise ValueError("the no-allocation launch takes no workspace")
+        if num_sms > NOALLOC_MAX_PROGRAMS:
+            raise ValueError(f"the no-allocation launch takes at most {NOALLOC_MAX_PROGRAMS} programs")
+        forced = split_k > 1 or split_k == SPLIT_STREAM_K
+        if forced and BLK_M * BLK_N > NOALLOC_MAX_TILE_ELEMS:
+            raise ValueError(f"a forced split of K needs tiles of at most {NOALLOC_MAX_TILE_ELEMS} elements here")
+        args = _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M,
+                               BLK_N, BLK_K, gsize_m, epilogue, phase, notify, num_xcds, scope, variant,
+                               mm_begin_timestamp, mm_end_timestamp, status, spin_timeout_ticks, None, None, 0)
+        args.split_k = split_k
+        launch = _native.lib().iris_gemm_launch_noalloc
+    else:
+        args = _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M,
+                               BLK_N, BLK_K, gsize_m, epilogue, phase, notify, num_xcds, scope, variant,
+                               mm_begin_timestamp, mm_end_timestamp, status, spin_timeout_ticks, partials, locks,
+                               split_k)
+        launch = _native.lib().iris_gemm_launch
     stream = torch.cuda.current_stream(a.device).cuda_stream
     with torch.cuda.device(a.device):
-        err = _native.lib().iris_gemm_launch(ctypes.byref(args), stream)
+        err = launch(ctypes.byref(args), stream)
     if err == _native.HIP_ERROR_INVALID_VALUE:
         raise ValueError(
             "iris_gemm_launch rejected the arguments (shape, strides, dtypes, grid or rank layout it does not take)"

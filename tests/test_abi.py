@@ -33,7 +33,7 @@ def test_libraries_load_and_export_every_declared_symbol():
     lib = _native.lib()
     for name in _native.SIGNATURES:
         assert getattr(lib, name) is not None
-    assert lib.iris_amd_abi_version() == 3
+    assert lib.iris_amd_abi_version() == 4
     alloc = ctypes.CDLL(_native.ALLOCATOR_LIB_PATH)
     for name in _native.ALLOCATOR_SYMBOLS:
         assert getattr(alloc, name) is not None

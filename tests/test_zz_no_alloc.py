@@ -1,0 +1,93 @@
+"""``iris_gemm_launch_noalloc``: the launch whose split-K / stream-K / few-rows
+workspace is a device array inside the library.  Its output must equal, bit
+for bit, what ``iris_gemm_launch`` gives with a caller-provided workspace (the
+same kernels, the same plan, the same order of fp32 additions), on two calls
+in a row, the second with a smaller input (the array keeps the first call's
+contents)."""
+
+import pytest
+import torch
+
+from iris_amd import ops
+from oracle import iris_oracle as O
+
+from test_gemm_gpu import check_close, make_ab, to_heap
+
+pytestmark = pytest.mark.gpu
+
+
+def run_pair(shmem, M, N, K, BM, BN, grid, dtype, split_k, expect_split):
+    A, B = make_ab(M, N, K, dtype, seed=7 + M)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    partials = shmem.zeros((grid, BM * BN), dtype=torch.float32)
+    locks = shmem.zeros((grid,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+    args = lambda cg, flags: (a, b, None, cg, flags, hb, 0, 1, grid, BM, BN, 64, 2, ops.EPI_ALL_SCATTER)
+    cg_ws, cg_na = shmem.zeros((M, N), dtype=dtype), shmem.zeros((M, N), dtype=dtype)
+    f_ws, f_na = shmem.zeros((total,), dtype=torch.int32), shmem.zeros((total,), dtype=torch.int32)
+    got = ops.gemm_split_k(*args(cg_ws, f_ws), partials=partials, locks=locks, split_k=split_k)
+    assert got == expect_split, f"the plan under test: split {got}, expected {expect_split}"
+    ops.gemm_launch(*args(cg_ws, f_ws), partials=partials, locks=locks, split_k=split_k)
+    ops.gemm_launch(*args(cg_na, f_na), split_k=split_k, noalloc=True)
+    torch.cuda.synchronize()
+    check_close(cg_ws, O.shard_gemm(A, B, dtype), "workspace launch vs oracle")
+    assert torch.equal(cg_na.cpu().view(torch.int16), cg_ws.cpu().view(torch.int16)), "no-alloc differs from the workspace launch"
+    assert f_na.cpu().tolist() == f_ws.cpu().tolist() == [1] * total
+
+
+def test_noalloc_matches_the_workspace_launch_twice(shmem):
+    # split-K 8 on 64 x 64 tiles, then a smaller input with another split
+    run_pair(shmem, 100, 200, 1024, 64, 64, 256, torch.bfloat16, 8, 8)
+    run_pair(shmem, 40, 72, 512, 64, 64, 256, torch.bfloat16, 2, 2)
+    # stream-K on 128 x 128 tiles (the largest slot), then a smaller one
+    run_pair(shmem, 512, 768, 2048, 128, 128, 16, torch.bfloat16, ops.SPLIT_STREAM_K, ops.SPLIT_STREAM_K)
+    run_pair(shmem, 128, 128, 512, 64, 64, 4, torch.float16, ops.SPLIT_STREAM_K, ops.SPLIT_STREAM_K)
+
+
+def test_noalloc_few_rows_counters_and_launcher_choice(shmem):
+    # the few-rows kernel counts a tile's arrivals in the same array
+    dtype = torch.bfloat16
+    for M, N, K in ((16, 1376, 4096), (1, 512, 1376)):
+        A, B = make_ab(M, N, K, dtype)
+        a, b = to_heap(shmem, A), to_heap(shmem, B)
+        total = ops.cdiv(N, 256)
+        hb = shmem.get_heap_bases()
+        locks = shmem.zeros((256,), dtype=torch.int32)
+        cg_ws, cg_na = shmem.zeros((M, N), dtype=dtype), shmem.zeros((M, N), dtype=dtype)
+        f_ws, f_na = shmem.zeros((total,), dtype=torch.int32), shmem.zeros((total,), dtype=torch.int32)
+        common = lambda cg, f: (a, b, None, cg, f, hb, 0, 1, 256, 256, 256, 64, 4, ops.EPI_ALL_SCATTER)
+        assert ops.gemm_plan_name(*common(cg_ws, f_ws), locks=locks) == "few_rows_16xN"
+        ops.gemm_launch(*common(cg_ws, f_ws), locks=locks)
+        ops.gemm_launch(*common(cg_na, f_na), noalloc=True)
+        torch.cuda.synchronize()
+        check_close(cg_ws, O.shard_gemm(A, B, dtype))
+        assert torch.equal(cg_na.cpu().view(torch.int16), cg_ws.cpu().view(torch.int16))
+        assert f_na.cpu().tolist() == f_ws.cpu().tolist() == [1] * total
+
+
+def test_noalloc_limits_are_errors(shmem):
+    dtype = torch.bfloat16
+    A, B = make_ab(256, 256, 2048, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((256, 256), dtype=dtype)
+    flags = shmem.zeros((16,), dtype=torch.int32)
+    with pytest.raises(ValueError, match="at most 256 programs"):  # more programs than the array has slots
+        ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 512, 64, 64, 64, 2, ops.EPI_ALL_SCATTER, noalloc=True)
+    with pytest.raises(ValueError, match="forced split"):  # a forced split of a tile larger than a slot
+        ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 256, 256, 256, 64, 2, ops.EPI_ALL_SCATTER, split_k=2,
+                        noalloc=True)
+    # the same checks inside the library, past the Python wrapper
+    from iris_amd import _native
+    import ctypes
+
+    args = ops._fill_gemm_args(a, b, None, cg, flags, None, 0, 1, 256, 64, 64, 64, 2, ops.EPI_ALL_SCATTER,
+                               ops.PHASE_FUSED, True, 1, ops.SCOPE_AGENT, 0, None, None, None, 0)
+    args.num_sms = 512
+    assert _native.lib().iris_gemm_launch_noalloc(ctypes.byref(args), None) == _native.HIP_ERROR_INVALID_VALUE
+    args.num_sms, args.block_m, args.block_n, args.split_k = 256, 256, 256, 2
+    assert _native.lib().iris_gemm_launch_noalloc(ctypes.byref(args), None) == _native.HIP_ERROR_INVALID_VALUE
+    # without a forced split a large tile simply runs unsplit
+    ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 256, 256, 256, 64, 2, ops.EPI_ALL_SCATTER, noalloc=True)
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, dtype))
