@@ -88,7 +88,10 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 /* phases of IRIS_EPI_ONE_SHOT (bit mask) */
 #define IRIS_PHASE_PRODUCE 1 /* store partial tile + signal the other ranks  (:197-218) */
 #define IRIS_PHASE_CONSUME 2 /* wait for the tile's flag, reduce, store       (:220-271) */
-#define IRIS_PHASE_FUSED 3   /* both, in one program, as the reference kernel */
+#define IRIS_PHASE_FUSED 3   /* both, in one program and tile by tile, as the reference kernel: every rank's
+                              * launch must be on its device at the same time (a program waits for its peers) */
+#define IRIS_PHASE_TWO_KERNELS 7 /* both, as two kernels on the stream: the producer GEMM, then the reduce kernel
+                                  * (iris_one_shot_reduce_launch) behind it */
 
 /* flag scopes */
 #define IRIS_SCOPE_AGENT 0  /* all "ranks" live on this GPU */

@@ -20,7 +20,7 @@ DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 # epilogues (IRIS_EPI_*)
 EPI_ALL_SCATTER, EPI_ATOMIC_ADD, EPI_ONE_SHOT = 0, 1, 2
 # ONE_SHOT phases (IRIS_PHASE_*)
-PHASE_PRODUCE, PHASE_CONSUME, PHASE_FUSED = 1, 2, 3
+PHASE_PRODUCE, PHASE_CONSUME, PHASE_FUSED, PHASE_TWO_KERNELS = 1, 2, 3, 7
 # flag scopes (IRIS_SCOPE_*)
 SCOPE_AGENT, SCOPE_SYSTEM = 0, 1
 # special values of GemmArgs.variant (include/iris_amd.h)

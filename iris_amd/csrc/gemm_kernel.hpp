@@ -79,8 +79,16 @@ struct GemmKArgs {
   float* partials;
   int32_t* locks;
   int64_t partial_stride;
-  uint32_t* status;   // optional: IRIS_STATUS_SPIN_TIMEOUT when a wait for a partial gave up
+  uint32_t* status;   // optional: IRIS_STATUS_SPIN_TIMEOUT when a wait for a partial or a tile flag gave up
   uint64_t timeout;   // bound of that wait, 100 MHz ticks
+  // One-shot epilogue inside the program (the FUSED build of the kernel): once
+  // a tile's partial is stored and signalled, the program waits for the
+  // tile's flag on its own rank, sums the tile over all ranks' `out` buffers
+  // and stores the result to `cg`.
+  char* cg;
+  int64_t sgm, sgn;  // strides of `cg`, elements
+  int cg_dt;         // element type of `cg`
+  int fused_vec;     // 16-byte strips allowed on `out` and `cg` in the in-program reduce
 };
 
 template <int DT>
@@ -681,12 +689,123 @@ __device__ inline void add_partials(const GemmKArgs& p, f32x4 (&acc)[Cfg::IM][Cf
 }
 
 // ---------------------------------------------------------------------------
+// One-shot reduce of one tile inside the GEMM program
+// ---------------------------------------------------------------------------
+
+// c_global[tile] = cast(sum over ranks 0..ws-1, in that order, of C_r[tile]):
+// the tail of the reference program, gemm_one_shot_all_reduce.py:236-271.  The
+// whole group works on the tile; a lane moves one 16-byte strip per rank, lanes
+// run along a row, and RG ranks x UN rows are in flight per lane.  Absent ranks
+// of the last group read through an empty descriptor: zeros, which leave an
+// fp32 sum that started at +0 unchanged.  Loads are coherent at the flags'
+// scope by themselves (sc1 / sc0 sc1) and the result is written through, like
+// the reference's store with cache_modifier=".wt".
+template <int IN_DT, int NT, int UN, bool SYS>
+__device__ inline void fused_reduce_tile(const GemmKArgs& p, const Item& it, int tid) {
+  constexpr int IES = Vec<IN_DT>::ES, VE = Vec<IN_DT>::N;
+  constexpr int RG = 4;
+  constexpr int LAUX = SYS ? (AUX_NT | AUX_SC1 | AUX_SC0) : (AUX_NT | AUX_SC1);
+  constexpr int SAUX = SYS ? (AUX_SC1 | AUX_SC0) : AUX_SC1;
+  const int m0 = it.lm0, n0 = it.ln0;
+  const int rows = it.m_end - m0, cols = it.n_end - n0;
+  const int oes = dtype_size(p.cg_dt);
+  if (rows <= 0 || cols <= 0) return;
+  if (p.fused_vec && cols % VE == 0) {
+    const int cv = cols / VE;  // 16-byte strips per tile row
+    const int tpr = min(cv, NT), rpp = NT / tpr;
+    const int r0 = tid / tpr, cl = tid - r0 * tpr;
+    const uint32_t in_bytes = ((uint32_t)(rows - 1) * (uint32_t)p.som + cols) * IES;
+    const uint32_t out_bytes = ((uint32_t)(rows - 1) * (uint32_t)p.sgm + cols) * oes;
+    const int64_t in0 = ((int64_t)m0 * p.som + n0) * IES;
+    const __amdgpu_buffer_rsrc_t out_rs =
+        tile_rsrc((const IRIS_GLOBAL char*)p.cg + ((int64_t)m0 * p.sgm + n0) * oes, out_bytes);
+    for (int cc = 0; cc < cv; cc += tpr) {
+      const int c = cc + cl;
+      const bool live = r0 < rpp && c < cv;
+      for (int rb = 0; rb < rows; rb += rpp * UN) {
+        float acc[UN][VE];
+        uint32_t ioff[UN], ooff[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          const uint32_t row = rb + r0 + u * rpp;
+          ioff[u] = live ? (row * (uint32_t)p.som + c * VE) * IES : DEAD_OFFSET;
+          ooff[u] = live ? (row * (uint32_t)p.sgm + c * VE) * oes : DEAD_OFFSET;
+#pragma unroll
+          for (int e = 0; e < VE; ++e) acc[u][e] = 0.f;
+        }
+        for (int rk0 = 0; rk0 < p.ws; rk0 += RG) {
+          float v[RG][UN][VE];
+#pragma unroll
+          for (int g = 0; g < RG; ++g) {
+            const bool present = rk0 + g < p.ws;
+            const __amdgpu_buffer_rsrc_t rs =
+                tile_rsrc((const IRIS_GLOBAL char*)rank_ptr(p, p.out, present ? rk0 + g : p.cur_rank) + in0,
+                          present ? in_bytes : 0);
+#pragma unroll
+            for (int u = 0; u < UN; ++u) load_vec<IN_DT, LAUX>(rs, ioff[u], v[g][u]);
+          }
+#pragma unroll
+          for (int g = 0; g < RG; ++g)
+#pragma unroll
+            for (int u = 0; u < UN; ++u)
+#pragma unroll
+              for (int e = 0; e < VE; ++e) acc[u][e] += v[g][u][e];
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          if (p.cg_dt == IRIS_DTYPE_F32)
+            store_vec<IRIS_DTYPE_F32, VE, SAUX>(out_rs, ooff[u], acc[u]);
+          else if (p.cg_dt == IRIS_DTYPE_BF16)
+            store_vec<IRIS_DTYPE_BF16, VE, SAUX>(out_rs, ooff[u], acc[u]);
+          else
+            store_vec<IRIS_DTYPE_F16, VE, SAUX>(out_rs, ooff[u], acc[u]);
+        }
+      }
+    }
+  } else {
+    // any strides, alignment and widths: element by element
+    for (int idx = tid; idx < rows * cols; idx += NT) {
+      const int r = idx / cols, cidx = idx - r * cols;
+      const int64_t ioff = ((int64_t)(m0 + r) * p.som + (int64_t)(n0 + cidx) * p.son) * IES;
+      float acc = 0.f;
+      for (int rk = 0; rk < p.ws; ++rk) {
+        const IRIS_GLOBAL char* src = (const IRIS_GLOBAL char*)rank_ptr(p, p.out, rk) + ioff;
+        if constexpr (IN_DT == IRIS_DTYPE_F32) {
+          const unsigned int w = SYS ? __hip_atomic_load((const IRIS_GLOBAL unsigned int*)src, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_SYSTEM)
+                                     : __hip_atomic_load((const IRIS_GLOBAL unsigned int*)src, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_AGENT);
+          acc += __builtin_bit_cast(float, w);
+        } else {
+          const unsigned short h = SYS ? __hip_atomic_load((const IRIS_GLOBAL unsigned short*)src, __ATOMIC_RELAXED,
+                                                           __HIP_MEMORY_SCOPE_SYSTEM)
+                                       : __hip_atomic_load((const IRIS_GLOBAL unsigned short*)src, __ATOMIC_RELAXED,
+                                                           __HIP_MEMORY_SCOPE_AGENT);
+          acc += from16<IN_DT>(h);
+        }
+      }
+      IRIS_GLOBAL char* d = (IRIS_GLOBAL char*)p.cg + ((int64_t)(m0 + r) * p.sgm + (int64_t)(n0 + cidx) * p.sgn) * oes;
+      if (p.cg_dt == IRIS_DTYPE_F32)
+        store_through((IRIS_GLOBAL unsigned int*)d, __builtin_bit_cast(unsigned int, acc), SYS);
+      else if (p.cg_dt == IRIS_DTYPE_BF16)
+        store_through((IRIS_GLOBAL unsigned short*)d, to16<IRIS_DTYPE_BF16>(acc), SYS);
+      else
+        store_through((IRIS_GLOBAL unsigned short*)d, to16<IRIS_DTYPE_F16>(acc), SYS);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // The kernel
 // ---------------------------------------------------------------------------
 
 // SPLIT: the split-K build of the kernel (only launched with p.split_k > 1);
 // the plain build carries none of its code or state.
-template <class Cfg, int OP, int ODT, bool SPLIT = false>
+// FUSED: the one-shot epilogue as the reference program runs it
+// (gemm_one_shot_all_reduce.py:197-271): store the partial tile, signal the
+// other ranks, wait for the tile's own flag, reduce it over all ranks and
+// store the result, tile by tile, while other programs are in their K loops.
+template <class Cfg, int OP, int ODT, bool SPLIT = false, bool FUSED = false>
 __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::WPE, Cfg::WPE))) void
 gemm_persistent_kernel(const GemmKArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
@@ -742,7 +861,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
   // have completed.  Waiting for that right after issuing them would stall
   // the matrix cores, so the publication is deferred to the top of the next
   // K-step, where the whole group waits on its memory counter anyway.
-  const bool defer_publish = Cfg::DMA && nk > 0 && p.flag_mode != 0;
+  const bool defer_publish = !FUSED && Cfg::DMA && nk > 0 && p.flag_mode != 0;
   int pending_tile = -1;
   // 1: the pending tile's stores are exactly the FAST_STORES youngest memory
   // operations of this wave, so the next hand-over can wait for the loads
@@ -790,7 +909,39 @@ gemm_persistent_kernel(const GemmKArgs p) {
     }
     const bool fast = store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN,
                                               c_it.m_end, c_it.n_end, lane);
-    if (c_it.last_sub) {
+    if constexpr (FUSED) {
+      static_assert(!SPLIT && (OP == OP_STORE16 || OP == OP_STORE32), "the in-program reduce follows a plain store");
+      if (c_it.last_sub) {
+        constexpr int IN_DT = OP == OP_STORE32 ? IRIS_DTYPE_F32 : ODT;
+        IRIS_LDS int* slot = (IRIS_LDS int*)(lds + Cfg::S * Cfg::STAGE);  // wave 0's scratch, idle by now
+        IRIS_WAIT_VMCNT(0);  // this wave's stores of the partial tile have completed
+        __syncthreads();
+        int ok = 1;
+        if (p.ws > 1) {
+          if (tid == 0) {
+            publish_tile(p, c_it.tile_id);  // +1 on every other rank (:207-218)
+            *slot = wait_tile_flag((IRIS_GLOBAL int32_t*)(p.flags + c_it.tile_id), p.ws, p.sys != 0, p.timeout,
+                                   p.status)
+                        ? 1
+                        : 0;  // CAS(ws-1 -> 0) until it succeeds (:220-234), bounded
+          }
+          __syncthreads();
+          ok = *slot;
+        }
+        if (ok) {
+          // rows in flight per lane: what the registers hold next to the next tile's operand fragments
+          constexpr int UN = Cfg::IM * Cfg::IN * 4 > 64 ? 2 : 4;
+          if (p.sys)
+            fused_reduce_tile<IN_DT, Cfg::NT, UN, true>(p, c_it, tid);
+          else
+            fused_reduce_tile<IN_DT, Cfg::NT, UN, false>(p, c_it, tid);
+        }
+        __syncthreads();  // the slot is scratch again
+        if (p.ts_end && tid == 0)
+          __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + c_it.tile_id),
+                                 (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    } else if (c_it.last_sub) {
       if (defer_publish) {
         pending_tile = __builtin_amdgcn_readfirstlane(c_it.tile_id);
         // the count only holds for a tile that is a single compute tile

@@ -41,7 +41,8 @@ bool vec_ok(const void* base, int64_t stride_m, int64_t stride_n, int es) {
 struct Plan {
   const GemmKernelEntry* entry = nullptr;
   GemmKArgs k{};
-  int fused_reduce = 0;  // ONE_SHOT with the CONSUME phase: follow with the reduce kernel
+  int fused_reduce = 0;  // ONE_SHOT, CONSUME on its own or IRIS_PHASE_TWO_KERNELS: follow with the reduce kernel
+  int in_program = 0;    // ONE_SHOT, IRIS_PHASE_FUSED: the build of the kernel that reduces each tile itself
   // the few-rows kernel instead of a table entry, one workgroup per 16 columns
   GemmKernelFn skinny = nullptr;
   int skinny_grid = 0, skinny_grid_y = 1, skinny_lds = 0;
@@ -75,7 +76,7 @@ bool plan_few_rows(const iris_gemm_args& a, int op, bool dma_ok, Plan* plan) {
     room = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 &&
            (int64_t)m_blocks * n_blocks <= (int64_t)cus * per_cu;
   }
-  const bool ok = a.M <= SKINNY_MAX_ROWS && room && a.K > 0 && dma_ok &&
+  const bool ok = a.M <= SKINNY_MAX_ROWS && room && a.K > 0 && dma_ok && !plan->in_program &&
                   a.block_m >= a.M && (a.block_n % SKINNY_COLS) == 0 && !a.mm_begin_timestamp &&
                   !a.mm_end_timestamp && (a.split_k == 0 || a.split_k == 1) && counters &&
                   ((int64_t)SKINNY_ROWS * a.stride_am + a.K) * 2 < lim &&
@@ -94,7 +95,7 @@ bool plan_few_rows(const iris_gemm_args& a, int op, bool dma_ok, Plan* plan) {
 // Split-K and stream-K.  The owner of a tile waits for the programs that hold
 // its other parts, so every part needs a program of its own that is resident
 // at the same time: no more programs than the device has CUs.
-hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, GemmKArgs* kp) {
+hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool in_program, GemmKArgs* kp) {
   GemmKArgs& k = *kp;
   k.split_k = 1;
   k.split_q = k.split_r = 0;
@@ -106,6 +107,10 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, Gemm
   k.stream_k = 0;
   if (a.split_k < 0 && a.split_k != IRIS_GEMM_SPLIT_STREAM_K) return hipErrorInvalidValue;
   const int nk = (a.K + pick.bk - 1) / pick.bk;
+  if (in_program) {
+    // the program that computes a tile also reduces it: K is never shared out
+    return (a.split_k > 1 || a.split_k == IRIS_GEMM_SPLIT_STREAM_K) ? hipErrorInvalidValue : hipSuccess;
+  }
   if (a.split_k != 1 && a.partials && a.locks) {
     int cus = 0, dev = 0;
     const bool resident = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 && a.num_sms <= cus;
@@ -208,7 +213,9 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
       break;
     case IRIS_EPI_ONE_SHOT:
       if (!a.c || !a.c_global) return hipErrorInvalidValue;
-      if ((a.phase & ~IRIS_PHASE_FUSED) != 0 || a.phase == 0) return hipErrorInvalidValue;
+      if (a.phase != IRIS_PHASE_PRODUCE && a.phase != IRIS_PHASE_CONSUME && a.phase != IRIS_PHASE_FUSED &&
+          a.phase != IRIS_PHASE_TWO_KERNELS)
+        return hipErrorInvalidValue;
       out_dt = a.c_dtype;
       op = out_dt == IRIS_DTYPE_F32 ? OP_STORE32 : OP_STORE16;
       k.out = static_cast<char*>(a.c);
@@ -216,8 +223,17 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
       k.son = a.stride_cn;
       k.dest_all = 0;
       k.flag_mode = 2;
-      plan->fused_reduce = (a.phase & IRIS_PHASE_CONSUME) ? 1 : 0;
+      plan->in_program = a.phase == IRIS_PHASE_FUSED ? 1 : 0;
+      plan->fused_reduce = (a.phase == IRIS_PHASE_CONSUME || a.phase == IRIS_PHASE_TWO_KERNELS) ? 1 : 0;
       if (!(a.phase & IRIS_PHASE_PRODUCE)) return hipSuccess;  // consumer only: no GEMM
+      if (plan->in_program) {
+        const int gdt = a.c_global_dtype;
+        if (gdt != IRIS_DTYPE_F32 && gdt != IRIS_DTYPE_F16 && gdt != IRIS_DTYPE_BF16) return hipErrorInvalidValue;
+        k.cg = static_cast<char*>(a.c_global);
+        k.sgm = a.stride_cm_global;
+        k.sgn = a.stride_cn_global;
+        k.cg_dt = gdt;
+      }
       break;
     default:
       return hipErrorInvalidValue;
@@ -255,6 +271,15 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   k.total_tiles = k.num_pid_m * k.num_pid_n;
   k.sys = a.scope == IRIS_SCOPE_SYSTEM;
   k.vec_out = vec_ok(k.out, k.som, k.son, dtype_size(out_dt)) ? 1 : 0;
+  if (plan->in_program) {
+    // 16-byte strips in the in-program reduce: aligned rows on both sides, tile
+    // origins on strip boundaries, rows at least as long as the matrix is wide
+    // and 32-bit offsets inside a tile
+    const int ies = dtype_size(out_dt), oes = dtype_size(k.cg_dt), ve = 16 / ies;
+    k.fused_vec = k.vec_out && vec_ok(k.cg, k.sgm, k.sgn, oes) && a.block_n % ve == 0 && (a.block_n * oes) % 16 == 0 &&
+                  k.som >= a.N && k.sgm >= a.N && ((int64_t)a.block_m + 64) * k.som * ies < (1ll << 31) &&
+                  ((int64_t)a.block_m + 64) * k.sgm * oes < (1ll << 31);
+  }
 
   int count = 0;
   const GemmKernelEntry* list = entries_for(a.ab_dtype, op, &count);
@@ -307,6 +332,7 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
       if (fits(list[i]) && list[i].cm == 64 && list[i].cn == 64) pick = &list[i];
   }
   if (!pick) return hipErrorInvalidValue;
+  if (plan->in_program && !pick->fn_fused) return hipErrorInvalidValue;
   // compute tiles per logical tile; a matrix smaller than one logical tile
   // has nothing beyond its own edge
   const int span_m = a.block_m < a.M ? a.block_m : a.M, span_n = a.block_n < a.N ? a.block_n : a.N;
@@ -314,7 +340,7 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   k.sub_n = (span_n + pick->cn - 1) / pick->cn;
   plan->entry = pick;
 
-  const hipError_t err = plan_split(a, *pick, &k);
+  const hipError_t err = plan_split(a, *pick, plan->in_program != 0, &k);
   // (under stream-K every program has a run: the reference's XCD remap stays)
   if (err != hipSuccess || k.stream_k) return err;
   // Fewer (tile, part) items than programs: deal them to the XCDs evenly, in
@@ -375,6 +401,13 @@ using namespace iris_amd;
 
 namespace {
 
+// The build of the picked kernel that the plan launches.
+GemmKernelFn plan_fn(const Plan& plan) {
+  const GemmKernelEntry* e = plan.entry;
+  if (plan.in_program) return e->fn_fused;
+  return (plan.k.split_k > 1 || plan.k.stream_k) ? e->fn_split : e->fn;
+}
+
 // Enqueue what `plan` describes on `stream`.
 hipError_t run_plan(const Plan& plan, const iris_gemm_args& args, void* stream) {
   hipError_t err = hipSuccess;
@@ -393,14 +426,15 @@ hipError_t run_plan(const Plan& plan, const iris_gemm_args& args, void* stream) 
     if (err != hipSuccess) return err;
   } else if (plan.entry) {
     const GemmKernelEntry* e = plan.entry;
-    const GemmKernelFn fn = (plan.k.split_k > 1 || plan.k.stream_k) ? e->fn_split : e->fn;
+    const GemmKernelFn fn = plan_fn(plan);
     if (e->lds_bytes > 64 * 1024) {
       err = ensure_lds(fn, e->lds_bytes);
       if (err != hipSuccess) return err;
     }
     if (dbg())
-      std::fprintf(stderr, "[iris_amd] gemm %s M=%d N=%d K=%d tiles=%d grid=%d sub=%dx%d lds=%d\n", e->name, plan.k.M,
-                   plan.k.N, plan.k.K, plan.k.total_tiles, plan.k.num_sms, plan.k.sub_m, plan.k.sub_n, e->lds_bytes);
+      std::fprintf(stderr, "[iris_amd] gemm %s%s M=%d N=%d K=%d tiles=%d grid=%d sub=%dx%d lds=%d\n", e->name,
+                   plan.in_program ? "+reduce" : "", plan.k.M, plan.k.N, plan.k.K, plan.k.total_tiles, plan.k.num_sms,
+                   plan.k.sub_m, plan.k.sub_n, e->lds_bytes);
     hipLaunchKernelGGL(fn, dim3(plan.k.num_sms), dim3(e->threads), e->lds_bytes, s, plan.k);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
@@ -533,7 +567,7 @@ extern "C" int iris_gemm_kernel_info(const iris_gemm_args* args, int* n_regs, in
   if (n_spills) *n_spills = 0;
   if (!plan.entry && !plan.skinny) return hipSuccess;
   hipFuncAttributes attr;
-  err = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(plan.skinny ? plan.skinny : plan.entry->fn));
+  err = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(plan.skinny ? plan.skinny : plan_fn(plan)));
   if (err != hipSuccess) return err;
   if (n_regs) *n_regs = attr.numRegs;
   if (n_spills) *n_spills = static_cast<int>(attr.localSizeBytes);
@@ -555,7 +589,7 @@ extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t
   hipError_t err = make_plan(*args, &plan);
   if (err != hipSuccess) return err;
   std::snprintf(buf, len, "%s%s", plan.skinny ? "few_rows_16xN" : plan.entry ? plan.entry->name : "",
-                plan.entry && plan.k.stream_k ? "+stream_k" : "");
+                plan.entry && plan.k.stream_k ? "+stream_k" : plan.entry && plan.in_program ? "+reduce" : "");
   return hipSuccess;
 }
 

@@ -20,6 +20,7 @@ struct GemmKernelEntry {
   int lds_bytes;
   GemmKernelFn fn;
   GemmKernelFn fn_split;  // split-K build, or null
+  GemmKernelFn fn_fused;  // build with the one-shot reduce inside the program (store epilogues), or null
   const char* name;
 };
 
@@ -31,12 +32,21 @@ constexpr GemmKernelFn split_fn() {
     return nullptr;
 }
 
+template <class Cfg, int OP, int ODT>
+constexpr GemmKernelFn fused_fn() {
+  if constexpr (OP == OP_STORE16 || OP == OP_STORE32)
+    return &gemm_persistent_kernel<Cfg, OP, ODT, false, true>;
+  else
+    return nullptr;
+}
+
 template <class Cfg, int OP>
 constexpr GemmKernelEntry make_entry(const char* name) {
   constexpr int ODT = (OP == OP_STORE32 || OP == OP_ATOMIC32) ? IRIS_DTYPE_F32 : Cfg::DT;
   return GemmKernelEntry{Cfg::DT, OP,      Cfg::CM, Cfg::CN, Cfg::BK,        Cfg::WM,
                          Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::NT, Cfg::LDS_BYTES,
-                         &gemm_persistent_kernel<Cfg, OP, ODT, false>, split_fn<Cfg, OP, ODT>(), name};
+                         &gemm_persistent_kernel<Cfg, OP, ODT, false>, split_fn<Cfg, OP, ODT>(), fused_fn<Cfg, OP, ODT>(),
+                         name};
 }
 
 // The variants, in the launcher's order of preference: the first entry whose
@@ -79,6 +89,10 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP,    \
                                                   IRIS_GEMM_ODT(DT, OP), false>(const GemmKArgs); \
   IRIS_GEMM_INSTANTIATE_SPLIT_##SPLIT(DT, OP, CM, CN, BK, WM, WN, S, DMA)
+// the store epilogues' build with the one-shot reduce inside the program
+#define IRIS_GEMM_INSTANTIATE_FUSED(DT, OP, CM, CN, BK, WM, WN, S, DMA, SPLIT, NAME)           \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP, \
+                                                  IRIS_GEMM_ODT(DT, OP), false, true>(const GemmKArgs);
 
 #define IRIS_GEMM_DECLARE(TAG) const GemmKernelEntry* gemm_entries_##TAG(int* count);
 IRIS_GEMM_DECLARE(bf16_store16)

@@ -23,6 +23,7 @@ from ._native import (
     PHASE_CONSUME,
     PHASE_FUSED,
     PHASE_PRODUCE,
+    PHASE_TWO_KERNELS,
     SCOPE_AGENT,
     SCOPE_SYSTEM,
     VARIANT_FEW_ROWS,
@@ -49,6 +50,7 @@ __all__ = [
     "PHASE_PRODUCE",
     "PHASE_CONSUME",
     "PHASE_FUSED",
+    "PHASE_TWO_KERNELS",
     "SCOPE_AGENT",
     "SCOPE_SYSTEM",
 ]

@@ -187,3 +187,58 @@ def test_scatter_ready_flags_gate_a_concurrent_reader(shmem, two_streams, scope)
     assert torch.equal(on(cg, 1)[:, NL:].cpu(), cg[:, NL:].cpu())
     assert torch.equal(out.cpu(), cg[:, NL:].float().cpu() * 2), "reader saw a tile before its stores"
     assert flags.cpu().tolist() == [0] * total and on(flags, 1).cpu().tolist() == [1] * total
+
+
+@pytest.mark.parametrize("scope", [ops.SCOPE_AGENT, ops.SCOPE_SYSTEM])
+@pytest.mark.parametrize("M,N,K,BM,BN,partial_dtype", [
+    (4096, 4096, 512, 256, 256, torch.float32),   # 256 tiles, two per program, one compute tile each
+    (4096, 4096, 512, 256, 256, torch.bfloat16),
+    (2048, 3072, 1024, 128, 128, torch.float32),  # 384 tiles, three per program
+    (1000, 1160, 328, 128, 128, torch.bfloat16),  # ragged M, N and K; 16-byte strips still fit
+    (520, 388, 264, 64, 64, torch.float32),       # ragged, 63 tiles on 128 programs
+    (300, 250, 136, 128, 64, torch.float32),      # N no multiple of four: the element-wise reduce
+])
+def test_one_shot_inside_the_program_two_ranks_side_by_side(shmem, two_streams, M, N, K, BM, BN, partial_dtype,
+                                                            scope):
+    """IRIS_PHASE_FUSED, the reference program's own order
+    (gemm_one_shot_all_reduce.py:197-271): each program stores its partial
+    tile, signals the other rank, waits for the tile's flag on its own rank,
+    sums the tile over both ranks and stores it, tile by tile.  Two ranks of
+    128 programs each share the 256 CUs, one stream per rank."""
+    ws, G = 2, 6
+    dtype = torch.bfloat16
+    A, B = make_ab(M, N, K * ws, dtype, scale=0.05, seed=M + N)
+    a_full, b_full = to_heap(shmem, A), to_heap(shmem, B)
+    c = shmem.zeros((M, N), dtype=partial_dtype)
+    cg = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    hb = shmem.get_heap_bases()
+    on = shmem.on_rank
+    for r in range(ws):
+        for t in (c, cg, flags):
+            on(t, r).zero_()
+
+    def launch(r):
+        args = (a_full[:, r * K:(r + 1) * K], b_full[r * K:(r + 1) * K, :], on(c, r), on(cg, r), on(flags, r), hb, r,
+                ws, 128, BM, BN, 64, G, ops.EPI_ONE_SHOT)
+        kw = dict(phase=ops.PHASE_FUSED, num_xcds=8)
+        assert ops.gemm_plan_name(*args, **kw).endswith("+reduce")
+        ops.gemm_launch(*args, status=status, spin_timeout_ticks=HALF_SECOND, scope=scope, **kw)
+
+    torch.cuda.synchronize()
+    for r, s in enumerate(two_streams):
+        with torch.cuda.stream(s):
+            launch(r)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0, "a program gave up waiting for its peer"
+    partials = torch.stack([on(c, r).cpu() for r in range(ws)])
+    shards = O.k_shards(A, B, ws)
+    for r in range(ws):
+        check_close(partials[r], O.shard_gemm(*shards[r], partial_dtype), f"partial of rank {r}")
+    want = O.one_shot_reduce(partials, dtype)
+    for r in range(ws):
+        assert torch.equal(on(cg, r).cpu(), want), f"rank {r}: not the rank-ordered sum of the partials"
+        assert on(flags, r).cpu().tolist() == [0] * total  # every flag went up once and was consumed
+    check_close(cg, O.one_shot_all_reduce(shards, partial_dtype, dtype), "vs closed form")

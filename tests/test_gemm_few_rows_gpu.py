@@ -144,11 +144,14 @@ def test_one_shot_producer_and_reduce(shmem, pdtype):
         assert not shmem.on_rank(flags, r).any()
 
 
+@pytest.mark.parametrize("phase", [ops.PHASE_TWO_KERNELS, ops.PHASE_FUSED])
 @pytest.mark.parametrize("ws", [1, 4])
-def test_one_shot_fused_phase(shmem, ws):
-    """PHASE_FUSED: the few-rows producer and the reduce kernel behind it on
-    the same stream.  With one GPU playing every rank the other ranks' partials
-    and signals are put in place first, then the last rank runs fused."""
+def test_one_shot_fused_phase(shmem, ws, phase):
+    """PHASE_TWO_KERNELS: the few-rows producer and the reduce kernel behind it
+    on the same stream.  PHASE_FUSED reduces inside the program, which the
+    persistent kernels do: the launch stays with them.  With one GPU playing
+    every rank the other ranks' partials and signals are put in place first,
+    then the last rank runs both phases."""
     M, N, BM, BN, G, dtype = 9, 272, 16, 64, 3, torch.bfloat16
     K = 192 * ws
     A, B = make_ab(M, N, K, dtype, scale=0.05)
@@ -168,8 +171,11 @@ def test_one_shot_fused_phase(shmem, ws):
     for r in range(ws):
         args = (ah[:, r * kk:(r + 1) * kk], bh[r * kk:(r + 1) * kk, :], shmem.on_rank(part, r), shmem.on_rank(out, r),
                 shmem.on_rank(flags, r), hb, r, ws, 256, BM, BN, 64, G, ops.EPI_ONE_SHOT)
-        kw = dict(phase=ops.PHASE_FUSED if r == last else ops.PHASE_PRODUCE, locks=shmem.on_rank(locks, r))
-        assert ops.gemm_plan_name(*args, **kw) == FEW
+        kw = dict(phase=phase if r == last else ops.PHASE_PRODUCE, locks=shmem.on_rank(locks, r))
+        if r == last and phase == ops.PHASE_FUSED:
+            assert ops.gemm_plan_name(*args, **kw).endswith("+reduce")
+        else:
+            assert ops.gemm_plan_name(*args, **kw) == FEW
         ops.gemm_launch(*args, **kw)
     torch.cuda.synchronize()
     check_close(shmem.on_rank(out, last), O.one_shot_all_reduce(shards, torch.float32, dtype), "fused result")

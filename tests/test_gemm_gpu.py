@@ -250,8 +250,9 @@ def test_atomic_add_ragged_and_on_every_rank(shmem):
 
 
 # --------------------------------------------------------------------------- one-shot
+@pytest.mark.parametrize("phase", [ops.PHASE_FUSED, ops.PHASE_TWO_KERNELS])  # reduce in the program / behind it
 @pytest.mark.parametrize("partial_dtype", [torch.bfloat16, torch.float32])
-def test_one_shot_fused_single_rank(shmem, partial_dtype):
+def test_one_shot_fused_single_rank(shmem, partial_dtype, phase):
     """world_size 1: store the tile to C, no flag traffic, c_global = cast(C)."""
     M, N, K = 384, 320, 192
     dtype = torch.bfloat16
@@ -262,7 +263,7 @@ def test_one_shot_fused_single_rank(shmem, partial_dtype):
     total = ops.cdiv(M, 128) * ops.cdiv(N, 64)
     flags = shmem.zeros((total,), dtype=torch.int32)
     ops.gemm_launch(a, b, c, cg, flags, shmem.get_heap_bases(), 0, 1, 8, 128, 64, 64, 6, ops.EPI_ONE_SHOT,
-                    phase=ops.PHASE_FUSED)
+                    phase=phase)
     torch.cuda.synchronize()
     check_close(c, O.shard_gemm(A, B, partial_dtype), "partial")
     assert torch.equal(cg.cpu(), O.one_shot_reduce(c.cpu()[None], dtype))  # bit-exact given the partial
@@ -317,7 +318,8 @@ def test_one_shot_all_reduce_virtual_ranks(shmem, ws, partial_dtype):
     assert int(status.item()) == 0
 
 
-def test_fused_phase_with_peers_missing_times_out_and_exits(shmem):
+@pytest.mark.parametrize("phase", [ops.PHASE_FUSED, ops.PHASE_TWO_KERNELS])
+def test_fused_phase_with_peers_missing_times_out_and_exits(shmem, phase):
     """A rank whose peers never signal: the bounded wait gives up, reports it
     and skips the reduce; the kernel still drains."""
     M, N, K, ws = 128, 128, 64, 2
@@ -331,7 +333,7 @@ def test_fused_phase_with_peers_missing_times_out_and_exits(shmem):
         shmem.on_rank(flags, r).zero_()
     status = torch.zeros(1, dtype=torch.int32, device="cuda")
     ops.gemm_launch(a, b, c, cg, flags, shmem.get_heap_bases(), 0, ws, 4, 64, 64, 64, 1, ops.EPI_ONE_SHOT,
-                    phase=ops.PHASE_FUSED, status=status, spin_timeout_ticks=2000)  # 20 us
+                    phase=phase, status=status, spin_timeout_ticks=2000)  # 20 us
     torch.cuda.synchronize()
     assert int(status.item()) == 1
     assert float((cg.float() - 5).abs().max()) == 0.0  # nothing was reduced
