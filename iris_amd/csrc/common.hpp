@@ -199,6 +199,10 @@ __device__ inline void block_barrier_raw() {
 
 __host__ __device__ inline int dtype_size(int dt) { return dt == IRIS_DTYPE_F32 ? 4 : 2; }
 
+// CU count of the current device, asked of the runtime once per device
+// (launchers consult it on every call); 256 when it cannot be read.
+int current_cu_count();
+
 // ---- scoped atomics on flags -----------------------------------------------
 
 __device__ inline void flag_add_release(IRIS_GLOBAL int32_t* p, int v, bool sys) {

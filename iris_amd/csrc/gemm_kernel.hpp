@@ -701,11 +701,14 @@ __device__ inline void add_partials(const GemmKArgs& p, f32x4 (&acc)[Cfg::IM][Cf
 // scope by themselves (sc1 / sc0 sc1) and the result is written through, like
 // the reference's store with cache_modifier=".wt".
 template <int IN_DT, int NT, int UN, bool SYS>
-__device__ inline void fused_reduce_tile(const GemmKArgs& p, const Item& it, int tid) {
+__device__ inline void fused_reduce_tile(const GemmKArgs& p, const Item& it, int tid) {  // tid: by value
   constexpr int IES = Vec<IN_DT>::ES, VE = Vec<IN_DT>::N;
   constexpr int RG = 4;
   constexpr int LAUX = SYS ? (AUX_NT | AUX_SC1 | AUX_SC0) : (AUX_NT | AUX_SC1);
   constexpr int SAUX = SYS ? (AUX_SC1 | AUX_SC0) : AUX_SC1;
+  // (opaque, so that the lane's offsets are computed here and not kept in
+  // registers across the K loop)
+  asm volatile("" : "+v"(tid));
   const int m0 = it.lm0, n0 = it.ln0;
   const int rows = it.m_end - m0, cols = it.n_end - n0;
   const int oes = dtype_size(p.cg_dt);
@@ -929,8 +932,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
           ok = *slot;
         }
         if (ok) {
-          // rows in flight per lane: what the registers hold next to the next tile's operand fragments
-          constexpr int UN = Cfg::IM * Cfg::IN * 4 > 64 ? 2 : 4;
+          // rows in flight per lane (the accumulators' registers are free by now)
+          constexpr int UN = 4;
           if (p.sys)
             fused_reduce_tile<IN_DT, Cfg::NT, UN, true>(p, c_it, tid);
           else

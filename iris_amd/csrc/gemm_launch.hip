@@ -71,10 +71,8 @@ bool plan_few_rows(const iris_gemm_args& a, int op, bool dma_ok, Plan* plan) {
                         (a.locks && k.total_tiles <= a.num_sms);
   bool room = true;
   if (m_blocks > 1) {
-    int cus = 0, dev = 0;
     const int per_cu = 160 * 1024 / skinny_lds_bytes(un) > 4 ? 4 : 160 * 1024 / skinny_lds_bytes(un);
-    room = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 &&
-           (int64_t)m_blocks * n_blocks <= (int64_t)cus * per_cu;
+    room = (int64_t)m_blocks * n_blocks <= (int64_t)current_cu_count() * per_cu;
   }
   const bool ok = a.M <= SKINNY_MAX_ROWS && room && a.K > 0 && dma_ok && !plan->in_program &&
                   a.block_m >= a.M && (a.block_n % SKINNY_COLS) == 0 && !a.mm_begin_timestamp &&
@@ -112,8 +110,7 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
     return (a.split_k > 1 || a.split_k == IRIS_GEMM_SPLIT_STREAM_K) ? hipErrorInvalidValue : hipSuccess;
   }
   if (a.split_k != 1 && a.partials && a.locks) {
-    int cus = 0, dev = 0;
-    const bool resident = hipGetDevice(&dev) == hipSuccess && iris_hip_cu_count(dev, &cus) == 0 && a.num_sms <= cus;
+    const bool resident = a.num_sms <= current_cu_count();
     const bool possible = resident && pick.splitk && pick.fn_split && k.sub_m == 1 && k.sub_n == 1 &&
                           a.partials_slot_elems >= (int64_t)pick.cm * pick.cn &&
                           (reinterpret_cast<uintptr_t>(a.partials) & 15) == 0 && (a.partials_slot_elems % 4) == 0;

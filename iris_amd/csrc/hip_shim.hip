@@ -6,7 +6,21 @@
 #include <cstdio>
 #include <cstring>
 
-#include "../../include/iris_amd.h"
+#include "common.hpp"
+
+namespace iris_amd {
+
+int current_cu_count() {
+  static int cached[64] = {};
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] > 0) return cached[dev];
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 256;
+  cached[dev] = cus;
+  return cus;
+}
+
+}  // namespace iris_amd
 
 extern "C" {
 

@@ -57,17 +57,6 @@ ReduceFn pick(int in_dt, int out_dt, int ws, int variant, bool sys, bool rows) {
   return nullptr;
 }
 
-// CU count of the current device, looked up once per device
-int current_cu_count() {
-  static int cached[64] = {};
-  int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] > 0) return cached[dev];
-  if (iris_hip_cu_count(dev, &cus) != 0 || cus <= 0) return 256;
-  cached[dev] = cus;
-  return cus;
-}
-
 bool valid_dtype(int dt) { return dt == IRIS_DTYPE_F32 || dt == IRIS_DTYPE_F16 || dt == IRIS_DTYPE_BF16; }
 
 }  // namespace

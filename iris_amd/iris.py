@@ -34,9 +34,14 @@ _TORCH_TYPESTR = "|i1"
 
 
 class _DeviceBytes:
-    """Zero-copy window on raw device memory for ``torch.as_tensor``."""
+    """Zero-copy window on raw device memory for ``torch.as_tensor``, and the
+    owner of that memory: torch keeps a reference to this object for as long as
+    any tensor views the storage, and the allocation is released when the last
+    of them is gone (the reference's pool is a torch tensor with the same
+    lifetime, iris/iris.py:48)."""
 
-    def __init__(self, ptr: int, nbytes: int):
+    def __init__(self, ptr: int, nbytes: int, owns: bool = False):
+        self._ptr = ptr if owns else None
         self.__cuda_array_interface__ = {
             "shape": (nbytes,),
             "typestr": _TORCH_TYPESTR,
@@ -45,6 +50,16 @@ class _DeviceBytes:
             "version": 3,
         }
 
+    def __del__(self):
+        ptr, self._ptr = self._ptr, None
+        if ptr is None:
+            return
+        try:
+            _hip.device_synchronize()  # no kernel may still be using the heap
+            _hip.hip_free(ptr)
+        except Exception:  # interpreter shutdown: the driver reclaims the memory
+            pass
+
 
 def _finegrained_pool(nbytes: int, device: str) -> torch.Tensor:
     """int8[nbytes] on fine-grained device memory."""
@@ -52,7 +67,7 @@ def _finegrained_pool(nbytes: int, device: str) -> torch.Tensor:
         # every torch allocation is fine-grained in this mode (see __init__)
         return torch.empty(nbytes, device=device, dtype=torch.int8)
     ptr = _hip.malloc_fine_grained(nbytes)
-    return torch.as_tensor(_DeviceBytes(ptr.value, nbytes), device=device)
+    return torch.as_tensor(_DeviceBytes(ptr.value, nbytes, owns=True), device=device)
 
 
 class Iris:

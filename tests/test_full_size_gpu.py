@@ -3,11 +3,9 @@
 reduce of eight fp32 [8192,8192] partials, the eight-shard atomic accumulate
 into fp32 [4096,4096], and the decoder-shaped shards for 1 ... 2048 rows.
 
-The full fp32 product is too much for the CPU oracle inside a test, so the
-GEMM is checked against the oracle on sampled rows and columns (every tile is
-crossed by some of them), against a column-sum identity over the whole
-matrix, and flag for flag.  The reduce is compared with the oracle bit for
-bit over the whole matrix.
+Every output element is compared with the oracle: the GEMMs within rtol /
+atol 1e-2 of the fp32-accumulated product, flags one by one, the reduce bit
+for bit.
 """
 
 import pytest
@@ -42,19 +40,8 @@ def test_headline_shard_gemm(shmem, G):
     torch.cuda.synchronize()
     assert flags.cpu().tolist() == [1] * total + [0]
 
-    # the oracle on 3 rows and 3 columns of every tile row / tile column
-    A, B = a.cpu(), b.cpu()
-    g = torch.Generator().manual_seed(7)
-    rows = torch.cat([torch.randint(0, BM, (3,), generator=g) + t * BM for t in range(M // BM)])
-    cols = torch.cat([torch.randint(0, BN, (3,), generator=g) + t * BN for t in range(N // BN)])
-    check_close(cg[rows].cpu(), O.shard_gemm(A[rows], B, dtype), "sampled rows")
-    check_close(cg[:, cols].cpu(), O.shard_gemm(A, B[:, cols], dtype), "sampled columns")
-
-    # whole matrix: 1^T C == (1^T A) B up to the rounding of C's 8192 addends per column
-    colsum = cg.float().sum(dim=0).cpu()
-    want = (A.float().sum(dim=0, keepdim=True) @ B.float()).squeeze(0)
-    bound = 8192 ** 0.5 * 2.0 ** -9 * cg.float().abs().max().item() * 6  # 6 sigma of independent bf16 roundings
-    assert (colsum - want).abs().max().item() < bound
+    # the whole [8192, 8192] product against the oracle
+    check_close(cg.cpu(), O.shard_gemm(a.cpu(), b.cpu(), dtype), "headline shard GEMM")
 
 
 def test_headline_reduce_of_eight_partials_is_bit_exact(shmem):
@@ -83,8 +70,8 @@ def test_headline_reduce_of_eight_partials_is_bit_exact(shmem):
 
 def test_atomic_accumulate_of_eight_shards_full_size(shmem):
     """Config 4: eight sequential bf16 K-shard GEMMs [4096,512] x [512,4096]
-    adding 256 tiles of 256x256 each into one fp32 C; the oracle on sampled
-    rows of every tile row."""
+    adding 256 tiles of 256x256 each into one fp32 C; the whole matrix
+    against the oracle."""
     M = N = 4096
     ks, shards, dtype = 512, 8, torch.bfloat16
     gen = torch.Generator(device="cuda").manual_seed(123)
@@ -97,15 +84,8 @@ def test_atomic_accumulate_of_eight_shards_full_size(shmem):
         ops.gemm_launch(a_full[:, i * ks:(i + 1) * ks], bt_full[:, i * ks:(i + 1) * ks].T, None, c, None,
                         shmem.get_heap_bases(), 0, 1, 256, 256, 256, 64, 6, ops.EPI_ATOMIC_ADD, num_xcds=8)
     torch.cuda.synchronize()
-    g = torch.Generator().manual_seed(11)
-    rows = torch.cat([torch.randint(0, 256, (4,), generator=g) + t * 256 for t in range(M // 256)])
     A, B = a_full.cpu(), bt_full.cpu().T
-    want = O.atomics_all_reduce(O.k_shards(A[rows], B, shards))
-    check_close(c[rows].cpu(), want, "sampled rows")
-    # whole matrix against the sampled-row check's own closed form: 1^T C == (1^T A) B
-    colsum = c.sum(dim=0).cpu()
-    ref = (A.float().sum(dim=0, keepdim=True) @ B.float()).squeeze(0)
-    assert torch.allclose(colsum, ref, rtol=1e-3, atol=1e-2)
+    check_close(c.cpu(), O.atomics_all_reduce(O.k_shards(A, B, shards)), "atomic accumulate")
 
 
 @pytest.mark.parametrize("M", [1, 16, 128, 512, 2048])

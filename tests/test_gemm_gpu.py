@@ -188,14 +188,21 @@ def test_unaligned_and_strided_output(shmem):
     check_close(c32, O.shard_gemm(A, B, None))
 
 
-@pytest.mark.parametrize("variant", range(1, 25))
-def test_every_tuning_variant_is_correct(shmem, variant):
+def _variant_names():
+    """The compiled kernel variants of the bf16 store path, asked of the
+    library (a host-side table: no device is touched)."""
+    names, v = [], 1
+    while (name := ops.gemm_variant_name(torch.bfloat16, False, False, v)) is not None:
+        names.append(name)
+        v += 1
+    assert len(names) >= 7  # the seven base tiles always exist
+    return names
+
+
+@pytest.mark.parametrize("variant,name", [(i + 1, n) for i, n in enumerate(_variant_names())])
+def test_every_tuning_variant_is_correct(shmem, variant, name):
     """Each compiled kernel variant of the bf16 store path, forced on a shape
     with ragged edges and several tiles per program."""
-    name = ops.gemm_variant_name(torch.bfloat16, False, False, variant)
-    if name is None:
-        assert variant > 7  # the seven base tiles always exist
-        pytest.skip("no such variant")
     dtype = torch.bfloat16
     M, N, K = 520, 776, 328
     A, B = make_ab(M, N, K, dtype, lda=336, ldb=344)
