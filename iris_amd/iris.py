@@ -9,11 +9,16 @@ behaviour.  What differs is underneath:
   zero-copy; the rest of the process keeps torch's own caching allocator.
   ``IRIS_AMD_PLUGGABLE_ALLOCATOR=1`` instead routes *every* torch allocation
   through the plug-in, as the reference does (iris/__init__.py:40-45);
-* there is no MPI.  A process is one rank; ``virtual_ranks=P`` carves the
-  allocation into P equal sub-heaps that play the P ranks' symmetric heaps on
-  this one GPU, so that ``heap_bases``/pointer translation, flags and partial
-  buffers behave exactly as with P processes.  An allocation advances every
-  sub-heap alike, which is the symmetric-heap property.
+* ranks come in two kinds.  Several processes (one rank each, started by
+  ``torchrun``, by an MPI launcher when mpi4py is there, or with
+  ``IRIS_AMD_RENDEZVOUS``; see ``_bootstrap.py``) exchange the IPC handles and
+  base addresses of their heaps through a host-side store and map each
+  other's heaps, as the reference does over MPI (iris/iris.py:53-77).  Or one
+  process plays every rank: ``virtual_ranks=P`` carves one allocation into P
+  equal sub-heaps, so that ``heap_bases``/pointer translation, flags and
+  partial buffers behave exactly as with P processes.  Either way an
+  allocation advances every rank's heap alike, which is the symmetric-heap
+  property.
 """
 
 from __future__ import annotations
@@ -24,7 +29,7 @@ import os
 import numpy as np
 import torch
 
-from . import _hip
+from . import _bootstrap, _hip
 
 STATS = True
 LOGGING = True
@@ -70,8 +75,18 @@ def _finegrained_pool(nbytes: int, device: str) -> torch.Tensor:
     return torch.as_tensor(_DeviceBytes(ptr.value, nbytes, owns=True), device=device)
 
 
+# hipIpcOpenMemHandle has been seen not to return for larger allocations
+_IPC_MAX_BYTES = (2 << 30) - 1
+
+
 class Iris:
-    def __init__(self, heap_size=1 << 30, *, virtual_ranks=None, cur_rank=0, _pool_factory=None):
+    def __init__(self, heap_size=1 << 30, *, virtual_ranks=None, cur_rank=0, _pool_factory=None, _comm=None):
+        self._peer_pools = None
+        if virtual_ranks is None and "IRIS_AMD_VIRTUAL_RANKS" not in os.environ and _pool_factory is None:
+            comm = _comm if _comm is not None else _bootstrap.init_comm()
+            if comm is not None and comm.size > 1:
+                self._init_multi_process(heap_size, comm)
+                return
         if virtual_ranks is None:
             virtual_ranks = int(os.environ.get("IRIS_AMD_VIRTUAL_RANKS", "1"))
         if virtual_ranks < 1 or not (0 <= cur_rank < virtual_ranks):
@@ -104,6 +119,47 @@ class Iris:
             device=self.device, dtype=torch.uint64
         )
 
+    def _init_multi_process(self, heap_size, comm):
+        """One rank per process: iris/iris.py:32-79 with the store (or MPI) of
+        ``_bootstrap`` in the place of the MPI helpers."""
+        if heap_size > _IPC_MAX_BYTES and os.environ.get("IRIS_AMD_ALLOW_LARGE_IPC") != "1":
+            raise ValueError(
+                f"heap_size {heap_size}: a heap that peers map through IPC must stay under 2 GiB here "
+                "(set IRIS_AMD_ALLOW_LARGE_IPC=1 to try a larger one)"
+            )
+        self.comm = comm
+        self.num_ranks, self.cur_rank = comm.size, comm.rank
+        self.heap_size, self.heap_offset, self.alignment = heap_size, 0, 1024
+        self.gpu_id = self.cur_rank % _hip.count_devices()
+        _hip.set_device(self.gpu_id)
+        self.device = f"cuda:{self.gpu_id}"
+        # peers keep this memory mapped: like the reference's pool it is never handed back
+        ptr = _hip.malloc_fine_grained(heap_size)
+        self._pool_all = torch.as_tensor(_DeviceBytes(ptr.value, heap_size), device=self.device)
+        self.memory_pool = self._pool_all
+        handle = _hip.get_ipc_handle(ptr, self.cur_rank)
+        comm.barrier()
+        all_handles = comm.allgather(handle)
+        all_bases = comm.allgather(np.array([ptr.value], dtype=np.uint64))
+        comm.barrier()
+        assert int(all_bases[self.cur_rank][0]) == ptr.value
+        self._bases, self._peer_pools = [], []
+        for rank in range(self.num_ranks):
+            if rank == self.cur_rank:
+                self._bases.append(ptr.value)
+                self._peer_pools.append(self._pool_all)
+            else:
+                mapped = _hip.open_ipc_handle(np.ascontiguousarray(all_handles[rank]), self.cur_rank)
+                self._bases.append(int(mapped))
+                self._peer_pools.append(torch.as_tensor(_DeviceBytes(int(mapped), heap_size), device=self.device))
+        for r, b in enumerate(self._bases):
+            self.log_debug(f"GPU {r}: Heap base {hex(b)}")
+        comm.barrier()
+        self.heap_bases = torch.from_numpy(np.array(self._bases, dtype=np.uint64)).to(
+            device=self.device, dtype=torch.uint64
+        )
+        comm.barrier()
+
     # ------------------------------------------------------------------ logging
     def _say(self, message):
         print(f"[Iris] [{self.cur_rank}/{self.num_ranks}] {message}")
@@ -121,9 +177,11 @@ class Iris:
             self._say(message)
 
     def broadcast(self, source_rank, value):
-        # One process holds every rank, so the root's value is the caller's.
-        # (Callers pass (value, rank); the reference forwards the pair
-        # positionally to a (value, root) helper, iris/iris.py:93-94.)
+        # Callers pass (value, rank): the reference forwards the pair
+        # positionally to a (value, root) helper, iris/iris.py:93-94.  With
+        # one process holding every rank the root's value is the caller's.
+        if self.comm is not None:
+            return self.comm.broadcast_scalar(source_rank, value)
         return source_rank
 
     # --------------------------------------------------------------- allocation
@@ -242,9 +300,12 @@ class Iris:
         return self.heap_bases
 
     def barrier(self):
-        # all queued device work done; there is no other process to meet
+        # all queued device work done, then meet the other processes, if any
+        # (iris/iris.py:272-276)
         if self._pool_all.is_cuda:
             torch.cuda.synchronize()
+        if self.comm is not None:
+            self.comm.barrier()
 
     def get_device(self):
         return self.memory_pool.device
@@ -275,7 +336,10 @@ class Iris:
             raise RuntimeError("The tensor is not on the symmetric heap")
         off = tensor.data_ptr() - self._bases[self.cur_rank]
         es = tensor.element_size()
-        window = self._pool_all[rank * self.heap_size + off:(rank + 1) * self.heap_size]
+        if self._peer_pools is not None:  # one process per rank: the peer's heap as mapped here
+            window = self._peer_pools[rank][off:]
+        else:
+            window = self._pool_all[rank * self.heap_size + off:(rank + 1) * self.heap_size]
         typed = window[:(window.numel() // es) * es].view(tensor.dtype)
         return typed.as_strided(tensor.size(), tensor.stride())
 
