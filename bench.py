@@ -96,26 +96,30 @@ def timed_steps(fn, steps, warmup):
 
 
 def cpu_baseline():
-    """The oracle's shard GEMM (fp32 matmul + bf16 downcast) on the host cores,
-    on a bounded sample: the first 2048 rows of A against all of B."""
+    """The oracle on the host cores at the full sizes of the two headline
+    workloads: the shard GEMM (fp32 matmul + bf16 downcast of [8192,1024] x
+    [1024,8192]) and the rank-ordered sum of eight fp32 [8192,8192] partials.
+    About ten seconds in all."""
     import torch
 
     from oracle import iris_oracle as O
 
-    rows = 2048
     g = torch.Generator().manual_seed(123)
-    A = (torch.randn(rows, K_SHARD, generator=g) * 0.02).to(torch.bfloat16)
+    A = (torch.randn(M, K_SHARD, generator=g) * 0.02).to(torch.bfloat16)
     B = (torch.randn(N, K_SHARD, generator=g) * 0.02).to(torch.bfloat16).T
     O.shard_gemm(A, B, torch.bfloat16)  # warm-up
     times = []
-    t_end = time.perf_counter() + 12.0
+    t_end = time.perf_counter() + 6.0
     while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 20):
         t0 = time.perf_counter()
         O.shard_gemm(A, B, torch.bfloat16)
         times.append(time.perf_counter() - t0)
     med = statistics.median(times)
-    # the reduce phase of the same math: 8 fp32 partials [1024, 8192] summed in rank order -> bf16
-    parts = torch.randn(8, 1024, N, generator=g)
+    del A, B
+    # the reduce phase: 8 fp32 partials [8192, 8192] (2 GiB on the host) summed in rank order -> bf16
+    parts = torch.empty(8, M, N)
+    for r in range(8):
+        parts[r].normal_(generator=g)
     O.one_shot_reduce(parts, torch.bfloat16)
     rtimes = []
     for _ in range(3):
@@ -124,14 +128,15 @@ def cpu_baseline():
         rtimes.append(time.perf_counter() - t0)
     rmed = statistics.median(rtimes)
     return {
-        "reduce_GBps": round((parts.numel() * 4 + 1024 * N * 2) / rmed / 1e9, 2),
-        "reduce_sample": "oracle one_shot_reduce of 8 fp32 partials [1024,8192] -> bf16, 3 runs, median",
-        "value": 2.0 * rows * N * K_SHARD / med / 1e12,
+        "reduce_GBps": round((parts.numel() * 4 + M * N * 2) / rmed / 1e9, 2),
+        "reduce_sample": "oracle one_shot_reduce of 8 fp32 partials [8192,8192] -> bf16 (the whole workload), 3 runs, "
+                         "median",
+        "value": 2.0 * M * N * K_SHARD / med / 1e12,
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"oracle shard_gemm (torch fp32 matmul + bf16 cast) on A[:{rows}] x B, {len(times)} runs, median; "
-                  f"os.cpu_count()={os.cpu_count()}",
+        "sample": f"oracle shard_gemm (torch fp32 matmul + bf16 cast) on the whole A[8192,1024] x B[1024,8192], "
+                  f"{len(times)} runs, median; os.cpu_count()={os.cpu_count()}",
     }
 
 
@@ -182,9 +187,10 @@ def graph_ms(fn, per_graph=20, replays=20):
     return s.elapsed_time(e) / (per_graph * replays)
 
 
-def context_figures(a, b, c_global, flops):
-    """Two figures that put the headline number in context, measured the same
-    way (settled clocks, back-to-back launches):
+def context_figures(a, b, c_global, flops, gemm_on):
+    """Figures that put the headline number in context, measured the same
+    way (settled clocks, back-to-back launches; ``gemm_on(a, b)`` launches the
+    headline GEMM on other operands):
 
     * the vendor library's GEMM (torch.matmul -> hipBLASLt) on the same
       operands and output buffer, without flags;
@@ -202,6 +208,17 @@ def context_figures(a, b, c_global, flops):
     ms = steady_ms(lambda: torch.matmul(a, b, out=c_global))
     out["library_gemm"] = {"what": "torch.matmul (hipBLASLt) on the same operands, no tile flags",
                            "ms": round(ms, 5), "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
+    # the same two kernels on all-zero operands of the same shape and strides: nothing toggles in the matrix
+    # cores or on the way to them, the clocks stay up, and what is left is the kernels' structure
+    az = torch.zeros((a.shape[0], a.stride(0)), dtype=a.dtype, device=a.device)[:, :a.shape[1]]
+    bz = torch.zeros((b.shape[1], b.stride(1)), dtype=b.dtype, device=b.device)[:, :b.shape[0]].T
+    ms = steady_ms(lambda: gemm_on(az, bz))
+    out["gemm_on_zeros"] = {"what": "this kernel, all-zero operands", "ms": round(ms, 5),
+                            "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
+    ms = steady_ms(lambda: torch.matmul(az, bz, out=c_global))
+    out["library_gemm_on_zeros"] = {"what": "torch.matmul (hipBLASLt), all-zero operands", "ms": round(ms, 5),
+                                    "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
+    del az, bz
     groups, iters = 256, 4000
     sink = torch.empty(groups * 512, dtype=torch.float32, device="cuda")
     for name, operands in (("random N(0,0.02)", (torch.randn(32768, device="cuda") * 0.02).to(torch.bfloat16)),
@@ -250,6 +267,13 @@ def run_atomic(args, emit=True):
     ms = steady_ms(step, n=max(10, args.steps // 10))
     flops = 2.0 * Ma * Na * ks * shards
     updates = Ma * Na * shards
+    # what the chip takes when it does nothing else: one coalesced fp32 atomic add per element of the same C,
+    # eight passes (the kernel of the reference's atomic_add microbenchmark, examples/04_atomic_add)
+    def atomics_only():
+        for _ in range(shards):
+            ops.p2p_bench("atomic_add", c.view(-1), None, hb, 0, 0, 1, block_size=512)
+
+    ceil_ms = steady_ms(atomics_only, n=max(10, args.steps // 10))
     result = {
         "metric": "atomic-accumulate epilogue: 8 K-shard GEMMs into one fp32 C", "value": round(flops / ms / 1e9, 2),
         "unit": "TFLOP/s", "n_gpus": 1, "ms_per_step": round(ms, 5), "higher_is_better": True, "dtype": "bf16",
@@ -258,6 +282,10 @@ def run_atomic(args, emit=True):
                                "tiles into C[4096,4096] in the fine-grained heap", "grid": grid},
         "atomic_updates_per_s": round(updates / (ms * 1e-3), 0),
         "atomic_GBps_at_4B": round(updates * 4 / (ms * 1e-3) / 1e9, 1),
+        "atomic_ceiling": {"what": "the same 8 x 16.8 M fp32 atomic adds on C with no GEMM in front "
+                                   "(iris_p2p_bench_launch, ATOMIC_ADD)",
+                           "ms": round(ceil_ms, 5), "updates_per_s": round(updates / (ceil_ms * 1e-3), 0),
+                           "frac_of_ceiling": round(ceil_ms / ms, 4)},
         "max_abs_err_vs_fp32": err,
     }
     if emit:
@@ -425,9 +453,12 @@ def main():
     hb = shmem.get_heap_bases()
     num_xcds = ops.default_num_xcds(shmem.get_cu_count(), GRID)
 
-    def gemm_step():
-        ops.gemm_launch(a, b, None, c_global, flags, hb, 0, 1, GRID, BLK_M, BLK_N, BLK_K, args.gsize_m,
+    def gemm_on(x, y):
+        ops.gemm_launch(x, y, None, c_global, flags, hb, 0, 1, GRID, BLK_M, BLK_N, BLK_K, args.gsize_m,
                         ops.EPI_ALL_SCATTER, notify=True, num_xcds=num_xcds, variant=args.variant)
+
+    def gemm_step():
+        gemm_on(a, b)
 
     flops = 2.0 * M * N * K_SHARD
     settle_launches = 0
@@ -441,7 +472,8 @@ def main():
     ms_per_step = wall / args.steps * 1e3
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     kernel_tflops = flops / (kernel_ms * 1e-3) / 1e12
-    assert int(flags.min().item()) == args.steps + args.warmup + settle_launches, "every tile publishes once per step"
+    assert int(flags.min().item()) == int(flags.max().item()) == args.steps + args.warmup + settle_launches, \
+        "every tile publishes once per step"
     regs, spills = ops.gemm_kernel_info(a, b, None, c_global, flags, hb, 0, 1, GRID, BLK_M, BLK_N, BLK_K,
                                         args.gsize_m, ops.EPI_ALL_SCATTER, num_xcds=num_xcds, variant=args.variant)
 
@@ -480,13 +512,18 @@ def main():
     }
 
     if not args.no_context:
-        result["context"] = context_figures(a, b, c_global, flops)
+        result["context"] = context_figures(a, b, c_global, flops, gemm_on)
 
     if not args.no_coldcache:
-        cold_ms = iris_amd.do_bench(gemm_step, shmem.barrier, lambda: None, n_warmup=5, n_repeat=20)
-        result["gemm_cold_cache"] = {"protocol": "do_bench: 256 MiB cache flush before every repetition, mean",
-                                     "ms": round(cold_ms, 5),
-                                     "tflops": round(flops / (cold_ms * 1e-3) / 1e12, 2)}
+        # the reference's own timing protocol (iris/util.py:62-104): every repetition starts behind a 256 MiB
+        # cache flush and a device synchronise, one event pair per launch
+        cold_ms = iris_amd.do_bench(gemm_step, shmem.barrier, lambda: None, n_warmup=10, n_repeat=50)
+        cold_tflops = flops / (cold_ms * 1e-3) / 1e12
+        result["gemm_cold_cache"] = {"protocol": "do_bench: 256 MiB cache flush before every repetition, mean of 50",
+                                     "ms": round(cold_ms, 5), "tflops": round(cold_tflops, 2),
+                                     "roofline": {"bound": "mfma", "achieved": round(cold_tflops, 2),
+                                                  "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                                  "frac": round(cold_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}}
 
     if not args.no_reduce:
         # reduce phase: 8 fp32 partials [8192,8192] (one per virtual rank) -> bf16
@@ -554,7 +591,8 @@ def main():
         keep = ("M", "kernel_up", "split_k_up", "gate_up_us", "gate_up_tflops", "gate_up_weight_GBps", "kernel_down",
                 "split_k_down", "down_us", "down_tflops", "reduce_us", "reduce_GBps")
         result["other_workloads"] = {
-            "atomic_accumulate": {k: at[k] for k in ("value", "unit", "ms_per_step", "atomic_updates_per_s", "config")},
+            "atomic_accumulate": {k: at[k] for k in ("value", "unit", "ms_per_step", "atomic_updates_per_s",
+                                                     "atomic_ceiling", "config")},
             "decoder_shards": {"config": dec["config"], "per_M": [{k: r[k] for k in keep} for r in dec["per_M"]]},
         }
 
