@@ -12,7 +12,14 @@ Differences, all forced by the hardware this runs on:
 * ``--virtual_ranks P`` (new) lets the one GPU play P ranks: the heap is
   carved into P symmetric sub-heaps and every rank's launch runs in turn.
   With the one-shot algorithm all producers run before the consumers, since
-  P programs that wait for each other cannot share one GPU.
+  P programs that wait for each other cannot share one GPU from one stream.
+* Started once per rank instead (``torchrun --nproc-per-node P``, or ``RANK``
+  / ``WORLD_SIZE`` with ``IRIS_AMD_RENDEZVOUS``; the reference uses
+  ``mpirun -np P``), every process is one rank with its own heap, mapped by
+  its peers over IPC, as in the reference.  The one-shot algorithm then runs
+  the reference's program as it is (produce, signal, wait, reduce, tile by
+  tile); on one GPU the ranks' kernels must be resident together, so
+  ``--gemm_sms`` is capped at the CU count divided by the ranks.
 """
 
 import argparse
@@ -81,10 +88,21 @@ def main(algorithm, argv=None):
     args = parse_args(defaults, argv)
 
     ranks = args["virtual_ranks"]
-    shmem = iris.iris(args["heap_size"], virtual_ranks=ranks)
+    # one process per rank when a launcher's environment says so, else this process plays `ranks` ranks
+    shmem = iris.iris(args["heap_size"], virtual_ranks=ranks) if ranks > 1 else iris.iris(args["heap_size"])
     rank = shmem.get_rank()
     world_size = shmem.get_num_ranks()
     cu_count = shmem.get_cu_count()
+    multi_process = shmem.comm is not None
+    played = [rank] if multi_process else list(range(world_size))
+    if multi_process:
+        matmul.scope = ops.SCOPE_SYSTEM  # peers are other processes (the reference's scope="sys")
+    if multi_process and algorithm == "one_shot_all_reduce" and iris._hip.count_devices() < world_size:
+        # ranks that share a GPU wait for each other's programs on it: all of them must fit at once
+        fit = max(8, (cu_count // world_size) // 8 * 8)
+        if args["gemm_sms"] > fit:
+            shmem.log(f"gemm_sms {args['gemm_sms']} -> {fit}: {world_size} ranks share the {cu_count} CUs of one GPU")
+            args["gemm_sms"] = fit
 
     datatype = DATATYPES[args["datatype"]]
     if datatype not in (torch.float16, torch.bfloat16):
@@ -107,11 +125,11 @@ def main(algorithm, argv=None):
     if k_split:
         ks = args["k"] // world_size
         args["k"] = ks
-        shards = [(A[:, r * ks:(r + 1) * ks], B[r * ks:(r + 1) * ks, :]) for r in range(world_size)]
+        shards = {r: (A[:, r * ks:(r + 1) * ks], B[r * ks:(r + 1) * ks, :]) for r in played}
     else:
         ns = args["n"] // world_size
         args["n"] = ns
-        shards = [(A, B[:, r * ns:(r + 1) * ns].clone()) for r in range(world_size)]
+        shards = {r: (A, B[:, r * ns:(r + 1) * ns].clone()) for r in played}
 
     for key, value in args.items():
         json_writer.add_field(key, value)
@@ -156,7 +174,7 @@ def main(algorithm, argv=None):
 
     def preamble():
         shmem.barrier()
-        for r in range(world_size):
+        for r in played:
             iris.memset_tensor(shmem.on_rank(tile_completed, r), 0)
         shmem.barrier()
 
@@ -168,14 +186,15 @@ def main(algorithm, argv=None):
         torch.cuda.nvtx.range_push("GEMM + Communication")
         with torch.cuda.stream(gemm_stream):
             timing["start_event"].record()
-            if algorithm == "one_shot_all_reduce" and world_size > 1:
-                for r in range(world_size):
+            if algorithm == "one_shot_all_reduce" and world_size > 1 and not multi_process:
+                for r in played:
                     launch(r, ops.PHASE_PRODUCE)
-                for r in range(world_size):
+                for r in played:
                     launch(r, ops.PHASE_CONSUME)
             else:
-                for r in range(world_size):
-                    launch(r)
+                # (one rank per process: 09 is the reference's single program, ops.PHASE_FUSED)
+                for r in played:
+                    launch(r, ops.PHASE_FUSED if algorithm == "one_shot_all_reduce" else None)
             timing["end_event"].record()
             timing["experiments"] += 1
         torch.cuda.nvtx.range_pop()
@@ -210,7 +229,7 @@ def main(algorithm, argv=None):
         def zeroing_preamble():
             preamble()
             if algorithm == "atomics_all_reduce":
-                for r in range(world_size):
+                for r in played:
                     shmem.on_rank(global_C, r).zero_()
                 shmem.barrier()
 

@@ -44,3 +44,39 @@ def test_one_shot_example_with_virtual_ranks_and_benchmark(tmp_path):
                           "--datatype", "fp16", "-v", "-b", "--virtual_ranks", "4", "--BLK_N", "128")
     assert data["success"] is True and data["world_size"] == 4 and data["k"] == 256
     assert data["triton_ms"] > 0 and data["triton_tflops"] > 0 and data["gemm_experiments"] == 126
+
+
+@pytest.mark.parametrize("example,extra", [
+    ("07_gemm_all_scatter", ["--BLK_M", "256", "--BLK_N", "64"]),
+    ("08_gemm_atomics_all_reduce", ["--BLK_M", "128", "--BLK_N", "128"]),
+    ("09_gemm_one_shot_all_reduce", ["--BLK_M", "256", "--BLK_N", "128"]),
+])
+def test_example_with_one_process_per_rank(tmp_path, example, extra):
+    """The reference's way of running the examples, `mpirun -np 2 python
+    benchmark.py`, with the launcher's environment in MPI's place: two
+    processes, two heaps mapped over IPC, and for 09 the reference's single
+    program (produce, signal, wait, reduce) on both ranks at once."""
+    out = tmp_path / "log.json"
+    procs = []
+    for r in range(2):
+        env = dict(os.environ, RANK=str(r), WORLD_SIZE="2", IRIS_AMD_RENDEZVOUS=f"file://{tmp_path / 'store'}",
+                   IRIS_AMD_RENDEZVOUS_TIMEOUT="120", HSA_ENABLE_IPC_MODE_LEGACY="0")
+        env.pop("IRIS_AMD_VIRTUAL_RANKS", None)
+        cmd = [sys.executable, "-u", os.path.join(ROOT, "examples", example, "benchmark.py"), "--output_file", str(out),
+               "--heap_size", str(1 << 28), "-m", "1024", "-n", "768", "-k", "1024", "--datatype", "bf16", "-v", *extra]
+        procs.append(subprocess.Popen(cmd, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                                      cwd=str(tmp_path)))
+    outs = []
+    try:
+        for p in procs:
+            outs.append(p.communicate(timeout=280)[0])
+    finally:
+        for p in procs:
+            if p.poll() is None:
+                p.kill()
+    for r, (p, text) in enumerate(zip(procs, outs)):
+        assert p.returncode == 0 and "Final C validation passed." in text, f"rank {r}:\n" + text[-3000:]
+    data = json.loads(out.read_text())
+    assert data["success"] is True and data["world_size"] == 2
+    if example.startswith("09"):
+        assert data["gemm_sms"] == 128  # two ranks share the 256 CUs
