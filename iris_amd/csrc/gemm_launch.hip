@@ -315,8 +315,10 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
       const GemmKernelEntry& e = list[i];
       if (!fits(e)) continue;
       if (a.block_m % e.cm != 0 || a.block_n % e.cn != 0) continue;
-      if (e.cm > 64 && e.cm >= 2 * a.M) continue;
-      if (e.cn > 64 && e.cn >= 2 * a.N) continue;
+      // (up to half a tall tile may be padding: its rows cost matrix-core time only, and
+      // the tall tiles are the ones whose K range can be shared out over idle programs)
+      if (e.cm > 64 && e.cm >= 4 * a.M) continue;
+      if (e.cn > 64 && e.cn >= 4 * a.N) continue;
       // An atomic epilogue is bound by the chip's atomic rate (329 G fp32
       // adds a second, 51 us for 4096 x 4096), and while a program walks its
       // K loop it sends none: with two half tiles per logical tile the
