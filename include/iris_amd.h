@@ -119,6 +119,10 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
  * locks; hipErrorInvalidValue when the launch cannot be cut this way.
  * iris_gemm_split_k reports this value when the launcher chose it itself. */
 #define IRIS_GEMM_SPLIT_STREAM_K (-1)
+/* iris_gemm_args.split_handover */
+#define IRIS_GEMM_HANDOVER_AUTO 0
+#define IRIS_GEMM_HANDOVER_OWNER 1
+#define IRIS_GEMM_HANDOVER_SLICED 2
 
 /*
  * Arguments of one persistent shard-GEMM launch.  It is the argument list of
@@ -165,7 +169,13 @@ typedef struct iris_gemm_args {
   int32_t* locks;       /* int32[num_sms], or NULL                                */
   int64_t partials_slot_elems; /* >= block_m * block_n                            */
   int32_t split_k;      /* 0 = let the launcher decide, 1 = never, n > 1 = force n, IRIS_GEMM_SPLIT_STREAM_K */
-  int32_t reserved0;
+  /* How the parts of a split tile meet (split-K proper; stream-K runs always
+   * hand over to the tile's first part): IRIS_GEMM_HANDOVER_AUTO lets the
+   * launcher decide, _OWNER: the first part adds the others' partials and runs
+   * the epilogue, _SLICED: every part leaves its partial, then sums and stores
+   * its share of the tile's rows.  Both add the partials in part order: the
+   * results are bit-identical. */
+  int32_t split_handover;
 } iris_gemm_args;
 
 /*

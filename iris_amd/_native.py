@@ -26,6 +26,7 @@ SCOPE_AGENT, SCOPE_SYSTEM = 0, 1
 # special values of GemmArgs.variant (include/iris_amd.h)
 VARIANT_FEW_ROWS, VARIANT_PERSISTENT = 1000, 1001
 SPLIT_STREAM_K = -1  # GemmArgs.split_k: stream-K
+HANDOVER_AUTO, HANDOVER_OWNER, HANDOVER_SLICED = 0, 1, 2  # GemmArgs.split_handover
 # status word (IRIS_STATUS_*)
 STATUS_OK, STATUS_SPIN_TIMEOUT = 0, 1
 
@@ -77,7 +78,7 @@ class GemmArgs(ctypes.Structure):
         ("locks", ctypes.c_void_p),
         ("partials_slot_elems", ctypes.c_int64),
         ("split_k", ctypes.c_int32),
-        ("reserved0", ctypes.c_int32),
+        ("split_handover", ctypes.c_int32),
     ]
 
 

@@ -76,6 +76,14 @@ struct GemmKArgs {
   // programs that follow it hold the rest and hand it over through
   // partials[program] / locks[program] as split-K parts do.
   int stream_k;
+  // Split-K with the sliced hand-over (split_k > 1 only): every part, the
+  // first included, leaves its partial tile in `partials` as a row-major
+  // fp32 matrix and raises locks[first slot]; once all have, part q sums rows
+  // [q CM / split_k, (q + 1) CM / split_k) over the parts in part order and
+  // runs the epilogue on them, so that no program does a whole tile's worth
+  // of serial work; locks[first slot + 1] counts the parts that are done, and
+  // the last one publishes the tile and re-arms both counters.
+  int sliced;
   float* partials;
   int32_t* locks;
   int64_t partial_stride;
@@ -688,6 +696,156 @@ __device__ inline void add_partials(const GemmKArgs& p, f32x4 (&acc)[Cfg::IM][Cf
     for (int b = 0; b < NB; ++b) acc[b / Cfg::IN][b % Cfg::IN] += __builtin_bit_cast(f32x4, v[g][b]);
 }
 
+// Sliced hand-over, second half: rows [r0, r1) of the tile whose parts lie in
+// slots slot0 .. slot0 + parts - 1 as row-major [CM, CN] fp32 matrices, summed
+// in part order (the order in which an owner would add them) and handed to
+// the epilogue operation: 16-byte strips of four columns, lanes along a row,
+// two strips a lane and eight parts in flight.  The whole group works on the
+// slice.  The destinations' heap bases come through ONE vector load, lane r
+// holding rank r's (a scalar load per rank and strip, each waited for before
+// the rank's stores could go out, cost more than everything else here).
+template <class Cfg, int OP, int ODT>
+__device__ inline void slice_epilogue(const GemmKArgs& p, const Item& it, int slot0, int parts, int r0, int r1,
+                                      int tid) {  // tid: by value
+  constexpr bool F32 = (OP == OP_STORE32 || OP == OP_ATOMIC32);
+  constexpr int ES = F32 ? 4 : 2;
+  constexpr int CN4 = Cfg::CN / 4, UN = 2, RG = 8;
+  // (opaque, so that the lane's offsets are computed here and not kept in
+  // registers across the K loop)
+  asm volatile("" : "+v"(tid));
+  const int nstrips = (r1 - r0) * CN4;
+  const int r_begin = p.dest_all ? 0 : p.cur_rank;
+  const int r_end = p.dest_all ? p.ws : p.cur_rank + 1;
+  const int rows_ok = it.m_end - it.m0, cols_ok = it.n_end - it.n0;
+  if (rows_ok <= 0 || cols_ok <= 0) return;
+  const int64_t tile_off = ((int64_t)it.m0 * p.som + (int64_t)it.n0 * p.son) * ES;
+  const uint32_t out_bytes = (uint32_t)(((int64_t)(rows_ok - 1) * p.som + cols_ok) * ES);
+  const bool vec = p.vec_out && ((int64_t)(Cfg::CM - 1) * p.som + Cfg::CN) * ES < ((int64_t)1 << 31);
+  // lane r of every wave: the heap base of rank r
+  const bool table = p.heap_bases != nullptr && r_end - r_begin > 1 && p.ws <= 64;
+  uint64_t lane_base = 0;
+  if (table && (tid & 63) < p.ws) lane_base = p.heap_bases[tid & 63];
+  for (int s0 = tid; s0 < nstrips; s0 += Cfg::NT * UN) {
+    f32x4 sum[UN];
+    int row[UN], col[UN];
+    uint32_t poff[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int idx = s0 + u * Cfg::NT;
+      const bool live = idx < nstrips;
+      row[u] = r0 + idx / CN4;
+      col[u] = (idx % CN4) * 4;
+      poff[u] = live ? (uint32_t)((row[u] * Cfg::CN + col[u]) * 4) : DEAD_OFFSET;
+      if (!live) row[u] = 0x40000000;  // past every edge
+      sum[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int q0 = 0; q0 < parts; q0 += RG) {
+      u32x4 v[RG][UN];
+#pragma unroll
+      for (int g = 0; g < RG; ++g) {
+        const bool present = q0 + g < parts;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(p.partials + (int64_t)(slot0 + (present ? q0 + g : 0)) * p.partial_stride), 0,
+            present ? Cfg::CM * Cfg::CN * 4 : 0, 0x00020000);
+#pragma unroll
+        for (int u = 0; u < UN; ++u)  // sc1: coherent at agent scope without a fence
+          v[g][u] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)poff[u], 0, AUX_SC1);
+      }
+#pragma unroll
+      for (int g = 0; g < RG; ++g)
+#pragma unroll
+        for (int u = 0; u < UN; ++u) sum[u] += __builtin_bit_cast(f32x4, v[g][u]);
+    }
+    const uint64_t cur_base = table ? (((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)(lane_base >> 32), p.cur_rank) << 32) |
+                                       (uint32_t)__builtin_amdgcn_readlane((int)lane_base, p.cur_rank))
+                                    : 0;
+    auto rank_dst = [&](int r) __attribute__((always_inline)) -> IRIS_GLOBAL char* {
+      if (table) {
+        const uint64_t rb = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)(lane_base >> 32), r) << 32) |
+                            (uint32_t)__builtin_amdgcn_readlane((int)lane_base, r);
+        return (IRIS_GLOBAL char*)translate(p.out, cur_base, rb) + tile_off;
+      }
+      return rank_ptr(p, p.out, r) + tile_off;
+    };
+    // what each strip needs, decided once: `ncols` valid columns; strips that
+    // are whole and may go out as one vector store have their offset, the
+    // others' offsets are parked out of range, so that the loop over the
+    // destinations is straight-line code
+    int ncols[UN];
+    uint32_t ooff[UN];
+    bool ragged = false;
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      ncols[u] = row[u] < rows_ok ? max(0, min(4, cols_ok - col[u])) : 0;
+      const bool whole = vec && ncols[u] == 4 && OP != OP_ATOMIC32;
+      ooff[u] = whole ? (uint32_t)(((int64_t)row[u] * p.som + col[u]) * ES) : DEAD_OFFSET;
+      ragged = ragged || (ncols[u] > 0 && !whole);
+    }
+    if constexpr (OP == OP_STORE32 || OP == OP_STORE16) {
+      u32x4 w32[UN];
+      u32x2 w16[UN];
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        w32[u] = __builtin_bit_cast(u32x4, sum[u]);
+        w16[u] = u32x2{pack2<ODT>(sum[u][0], sum[u][1]), pack2<ODT>(sum[u][2], sum[u][3])};
+      }
+      auto all_ranks = [&](auto aux_tag) __attribute__((always_inline)) {
+        constexpr int AUX = decltype(aux_tag)::value;
+#pragma nounroll
+        for (int r = r_begin; r < r_end; ++r) {
+          const __amdgpu_buffer_rsrc_t rs = tile_rsrc(rank_dst(r), out_bytes);
+#pragma unroll
+          for (int u = 0; u < UN; ++u) {
+            if constexpr (OP == OP_STORE32)
+              __builtin_amdgcn_raw_buffer_store_b128(w32[u], rs, (int)ooff[u], 0, AUX);
+            else
+              __builtin_amdgcn_raw_buffer_store_b64(w16[u], rs, (int)ooff[u], 0, AUX);
+          }
+        }
+      };
+      if (p.sys)
+        all_ranks(std::integral_constant<int, 17>{});
+      else
+        all_ranks(std::integral_constant<int, 16>{});
+    } else if constexpr (OP == OP_ATOMIC16) {
+#pragma nounroll
+      for (int r = r_begin; r < r_end; ++r) {
+        IRIS_GLOBAL char* dst = rank_dst(r);
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          if (ooff[u] == DEAD_OFFSET) continue;
+          atomic_add16_pair<ODT>((IRIS_GLOBAL unsigned int*)(dst + ooff[u]), pack2<ODT>(sum[u][0], sum[u][1]));
+          atomic_add16_pair<ODT>((IRIS_GLOBAL unsigned int*)(dst + ooff[u] + 4), pack2<ODT>(sum[u][2], sum[u][3]));
+        }
+      }
+    }
+    if (ragged) {
+      // ragged edge, odd strides or alignment, fp32 atomics: element by element
+#pragma nounroll
+      for (int r = r_begin; r < r_end; ++r) {
+        IRIS_GLOBAL char* dst = rank_dst(r);
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          if (ooff[u] != DEAD_OFFSET) continue;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (e >= ncols[u]) continue;
+            IRIS_GLOBAL char* d = dst + ((int64_t)row[u] * p.som + (int64_t)(col[u] + e) * p.son) * ES;
+            if constexpr (OP == OP_STORE32)
+              store_through((IRIS_GLOBAL unsigned int*)d, __builtin_bit_cast(unsigned int, sum[u][e]), p.sys != 0);
+            else if constexpr (OP == OP_STORE16)
+              store_through((IRIS_GLOBAL unsigned short*)d, to16<ODT>(sum[u][e]), p.sys != 0);
+            else if constexpr (OP == OP_ATOMIC32)
+              __hip_atomic_fetch_add((IRIS_GLOBAL float*)d, sum[u][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else
+              atomic_add16_cas<ODT>((IRIS_GLOBAL unsigned short*)d, from16<ODT>(to16<ODT>(sum[u][e])));
+          }
+        }
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // One-shot reduce of one tile inside the GEMM program
 // ---------------------------------------------------------------------------
@@ -887,6 +1045,54 @@ gemm_persistent_kernel(const GemmKArgs p) {
       pending_tile = -1;
     }
     if constexpr (SPLIT) {
+      if (p.sliced) {
+        // split-K proper: program pid is part pid % split_k of tile pid / split_k
+        const int parts = p.split_k;
+        const int slot0 = __builtin_amdgcn_readfirstlane((int)((unsigned)pid / (unsigned)parts) * parts);
+        const int part = pid - slot0;
+        IRIS_LDS int* okslot = (IRIS_LDS int*)(lds + Cfg::S * Cfg::STAGE);  // wave 0's scratch, idle here
+        {
+          // the partial as a row-major [CM, CN] fp32 matrix in slot `pid`, through
+          // the fp32 store epilogue (whole 128-byte lines, written through)
+          GemmKArgs q = p;
+          q.out = (char*)(p.partials + (int64_t)pid * p.partial_stride);
+          q.som = Cfg::CN;
+          q.son = 1;
+          q.dest_all = 0;
+          q.vec_out = 1;
+          q.sys = 0;
+          q.heap_bases = nullptr;
+          store_acc<Cfg, OP_STORE32, IRIS_DTYPE_F32>(q, acc, ws, wm * Cfg::TM, wn * Cfg::TN, Cfg::CM, Cfg::CN, lane);
+        }
+        IRIS_WAIT_VMCNT(0);  // this wave's part of the partial has been written
+        __syncthreads();
+        if (tid == 0) {
+          flag_add_relaxed((IRIS_GLOBAL int32_t*)(p.locks + slot0), 1, false);
+          *okslot = wait_tile_ready((IRIS_GLOBAL int32_t*)(p.locks + slot0), parts, false, p.timeout, p.status) ? 1 : 0;
+        }
+        __syncthreads();
+        const int ok = *okslot;
+        if (ok)
+          slice_epilogue<Cfg, OP, ODT>(p, c_it, slot0, parts, part * Cfg::CM / parts, (part + 1) * Cfg::CM / parts,
+                                       tid);
+        IRIS_WAIT_VMCNT(0);  // this wave's stores of the slice have completed
+        __syncthreads();     // (and okslot is scratch again)
+        if (tid == 0 && ok) {
+          IRIS_GLOBAL int32_t* done = (IRIS_GLOBAL int32_t*)(p.locks + slot0 + 1);
+          const int before = __hip_atomic_fetch_add(done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (before == parts - 1) {
+            // every slice is in memory: publish, and leave both counters at 0
+            if (p.flag_mode != 0) publish_tile(p, c_it.tile_id);
+            flag_add_relaxed(done, -parts, false);
+            flag_add_relaxed((IRIS_GLOBAL int32_t*)(p.locks + slot0), -parts, false);
+          }
+        }
+        if (p.ts_end && tid == 0)
+          __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + c_it.tile_id),
+                                 (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, sr, pid, c_item);
+        return;
+      }
       const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, c_item, nk);
       if (kr.part != 0) {
         // not the owner: leave the partial, raise the lock once every wave's

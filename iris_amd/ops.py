@@ -29,6 +29,9 @@ from ._native import (
     VARIANT_FEW_ROWS,
     VARIANT_PERSISTENT,
     SPLIT_STREAM_K,
+    HANDOVER_AUTO,
+    HANDOVER_OWNER,
+    HANDOVER_SLICED,
 )
 
 __all__ = [
@@ -229,7 +232,7 @@ def _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_s
 def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
                 gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, scope=SCOPE_AGENT, variant=0,
                 mm_begin_timestamp=None, mm_end_timestamp=None, status=None, spin_timeout_ticks=0, partials=None,
-                locks=None, split_k=0, noalloc=False):
+                locks=None, split_k=0, noalloc=False, split_handover=HANDOVER_AUTO):
     """Launch the persistent shard GEMM ``a @ b`` with a tile-publishing epilogue.
 
     ``partials`` / ``locks`` are the wrappers' ``P`` and ``locks`` buffers
@@ -237,7 +240,10 @@ def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size,
     programs splits each tile's K range over several programs, and a launch
     whose last round of tiles would leave many programs idle is cut into equal
     runs of K-steps (stream-K, ``split_k=SPLIT_STREAM_K`` to insist) (``split_k`` 0:
-    the launcher decides, 1: never, n: exactly n).
+    the launcher decides, 1: never, n: exactly n).  ``split_handover``: how the
+    parts of a split tile meet: ``HANDOVER_OWNER`` (the first part adds the
+    others' partials and stores the tile), ``HANDOVER_SLICED`` (every part sums
+    and stores its share of the rows) or ``HANDOVER_AUTO``; bit-identical results.
 
     ``noalloc=True`` goes through ``iris_gemm_launch_noalloc``: no workspace
     is passed, the library's own device array takes its place.
@@ -263,6 +269,7 @@ def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size,
                                mm_begin_timestamp, mm_end_timestamp, status, spin_timeout_ticks, partials, locks,
                                split_k)
         launch = _native.lib().iris_gemm_launch
+    args.split_handover = split_handover
     stream = torch.cuda.current_stream(a.device).cuda_stream
     with torch.cuda.device(a.device):
         err = launch(ctypes.byref(args), stream)

@@ -424,8 +424,10 @@ def split_workspace(shmem, grid, BM, BN):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_split_k_all_scatter(shmem, M, N, K, BM, BN, split_k, dtype):
     """A tile's K range shared by several programs: partials through the
-    workspace, the owner adds them, stores and publishes.  Twice in a row: the
-    locks are left re-armed."""
+    workspace; either the first part adds them, stores and publishes, or every
+    part sums and stores its share of the tile's rows and the last one to
+    finish publishes.  Twice in a row each way: the locks are left re-armed.
+    Both add the partials in part order, so the results are bit-identical."""
     A, B = make_ab(M, N, K, dtype)
     a, b = to_heap(shmem, A), to_heap(shmem, B)
     cg = shmem.zeros((M, N), dtype=dtype)
@@ -434,14 +436,21 @@ def test_split_k_all_scatter(shmem, M, N, K, BM, BN, split_k, dtype):
     grid = 256
     partials, locks = split_workspace(shmem, grid, BM, BN)
     want = O.shard_gemm(A, B, dtype)
-    for launch in (1, 2):
-        cg.zero_()
-        ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, grid, BM, BN, 64, 2, ops.EPI_ALL_SCATTER, partials=partials,
-                        locks=locks, split_k=split_k)
-        torch.cuda.synchronize()
-        check_close(cg, want, f"launch {launch}")
-        assert flags.cpu().tolist() == [launch] * total
-        assert int(locks.abs().max().item()) == 0
+    got = {}
+    launch = 0
+    for handover in (ops.HANDOVER_OWNER, ops.HANDOVER_SLICED, ops.HANDOVER_AUTO):
+        for again in (1, 2):
+            launch += 1
+            cg.zero_()
+            ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, grid, BM, BN, 64, 2, ops.EPI_ALL_SCATTER,
+                            partials=partials, locks=locks, split_k=split_k, split_handover=handover)
+            torch.cuda.synchronize()
+            check_close(cg, want, f"hand-over {handover}, launch {again}")
+            assert flags.cpu().tolist() == [launch] * total
+            assert int(locks.abs().max().item()) == 0
+        got[handover] = cg.cpu().clone()
+    assert torch.equal(got[ops.HANDOVER_OWNER].view(torch.int16), got[ops.HANDOVER_SLICED].view(torch.int16))
+    assert torch.equal(got[ops.HANDOVER_AUTO].view(torch.int16), got[ops.HANDOVER_SLICED].view(torch.int16))
 
 
 def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
@@ -609,20 +618,27 @@ def test_split_k_with_the_other_epilogues_and_virtual_ranks(shmem):
     c32 = shmem.zeros((M, N), dtype=torch.float32)
     for r in range(ws):
         shmem.on_rank(c32, r).zero_()
-    ops.gemm_launch(a, b, None, shmem.on_rank(c32, 1), None, hb, 1, ws, 256, 64, 64, 64, 2, ops.EPI_ATOMIC_ADD,
-                    partials=partials, locks=locks, split_k=8)
-    torch.cuda.synchronize()
-    for r in range(ws):
-        check_close(shmem.on_rank(c32, r), want32, f"atomic add on rank {r}")
+    for handover in (ops.HANDOVER_OWNER, ops.HANDOVER_SLICED):
+        for r in range(ws):
+            shmem.on_rank(c32, r).zero_()
+        ops.gemm_launch(a, b, None, shmem.on_rank(c32, 1), None, hb, 1, ws, 256, 64, 64, 64, 2, ops.EPI_ATOMIC_ADD,
+                        partials=partials, locks=locks, split_k=8, split_handover=handover)
+        torch.cuda.synchronize()
+        for r in range(ws):
+            check_close(shmem.on_rank(c32, r), want32, f"atomic add on rank {r}, hand-over {handover}")
+        assert int(locks.abs().max().item()) == 0
     part = shmem.zeros((M, N), dtype=torch.float32)
     out = shmem.zeros((M, N), dtype=dtype)
     flags = shmem.zeros((4,), dtype=torch.int32)
     for r in range(ws):
         shmem.on_rank(flags, r).zero_()
-    ops.gemm_launch(a, b, shmem.on_rank(part, 2), shmem.on_rank(out, 2), shmem.on_rank(flags, 2), hb, 2, ws, 256, 64,
-                    64, 64, 2, ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=partials, locks=locks, split_k=4)
-    torch.cuda.synchronize()
-    check_close(shmem.on_rank(part, 2), want32, "one-shot partial")
-    for r in range(ws):  # the producer signals every other rank once per tile
-        assert shmem.on_rank(flags, r).cpu().tolist() == [0 if r == 2 else 1] * 4
-    assert int(locks.abs().max().item()) == 0
+    for n, handover in enumerate((ops.HANDOVER_OWNER, ops.HANDOVER_SLICED), start=1):
+        shmem.on_rank(part, 2).zero_()
+        ops.gemm_launch(a, b, shmem.on_rank(part, 2), shmem.on_rank(out, 2), shmem.on_rank(flags, 2), hb, 2, ws, 256,
+                        64, 64, 64, 2, ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=partials, locks=locks,
+                        split_k=4, split_handover=handover)
+        torch.cuda.synchronize()
+        check_close(shmem.on_rank(part, 2), want32, f"one-shot partial, hand-over {handover}")
+        for r in range(ws):  # the producer signals every other rank once per tile
+            assert shmem.on_rank(flags, r).cpu().tolist() == [0 if r == 2 else n] * 4
+        assert int(locks.abs().max().item()) == 0
