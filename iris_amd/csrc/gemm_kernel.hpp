@@ -131,10 +131,14 @@ struct GemmCfg {
   static constexpr int A_LOADS = CM * CPR / NT, B_LOADS = CN * CPR / NT;
   static constexpr int L = A_LOADS + B_LOADS;
   static constexpr int KSUB = BK / 32;  // K-substeps (one MFMA depth) per stage
-  // Split-K is compiled into the tiles with at most 64 accumulator registers
-  // a lane: the exchange of partials needs registers the 128x64 wave tiles do
-  // not have to spare, and those tiles are picked for shapes that fill the chip.
-  static constexpr bool SPLITK = IM * IN * 4 <= 64 && KSUB % 2 == 0;
+  // Every LDS-DMA tile with two substeps a stage has a split-K build.  In the
+  // tiles with at most 64 accumulator registers a lane the first part of a tile
+  // can add the other parts' partials to its accumulators (which is also how
+  // stream-K runs hand over); the 128x64 wave tiles have no registers to spare
+  // for that exchange and only take the sliced hand-over, in which a part's
+  // accumulators are dead once its partial is written.
+  static constexpr bool SPLITK = DMA_ && KSUB % 2 == 0;
+  static constexpr bool SPLIT_OWNER = SPLITK && IM * IN * 4 <= 64;
   // Waves per SIMD the register budget is sized for: 256 registers a wave.
   static constexpr int WPE = 2;
   // wave-private epilogue scratch: 32 rows x TN 16-bit elements
@@ -1093,6 +1097,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
         if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, sr, pid, c_item);
         return;
       }
+      // (the tiles without the owner's way are only launched with the sliced one)
+      if constexpr (Cfg::SPLIT_OWNER) {
       const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, c_item, nk);
       if (kr.part != 0) {
         // not the owner: leave the partial, raise the lock once every wave's
@@ -1114,6 +1120,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       if (__syncthreads_and(ok)) {
         constexpr int GROUP = Cfg::IM * Cfg::IN * 4 <= 16 ? 4 : Cfg::IM * Cfg::IN * 4 <= 32 ? 2 : 1;
         for (int q = 1; q < parts; q += GROUP) add_partials<Cfg, GROUP>(p, acc, kr.slot, q, parts, tid);
+      }
       }
     }
     const bool fast = store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN,

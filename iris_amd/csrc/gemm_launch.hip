@@ -120,7 +120,8 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
     // A run of at least four steps keeps the parts of a tile few.
     const int64_t steps = (int64_t)k.total_tiles * nk;
     const int run = (int)(steps / a.num_sms);
-    const bool stream_ok = possible && run >= 4 && steps < ((int64_t)1 << 30) && (nk + run - 1) / run + 1 <= 32;
+    const bool stream_ok = possible && pick.split_owner && run >= 4 && steps < ((int64_t)1 << 30) &&
+                           (nk + run - 1) / run + 1 <= 32;
     if (a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
       if (!stream_ok) return hipErrorInvalidValue;
       k.stream_k = 1;
@@ -132,14 +133,17 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
       // K-steps a program walks through, unsplit
       const int rounds = (k.total_tiles + a.num_sms - 1) / a.num_sms;
       int walk = rounds * nk;
-      if (k.total_tiles * 2 <= a.num_sms && nk >= 32) {
+      if (k.total_tiles * 2 <= a.num_sms && nk >= 16) {
         // The hand-over of partials costs about as much as ten K-steps of a
-        // small tile, so only long K loops are split: as many parts as there
-        // are idle programs, at least four K-steps each.
+        // small tile: as many parts as there are idle programs, at least four
+        // K-steps each, and a K loop shorter than 32 steps is only split in
+        // four or more parts (measured on [M, 1376] x [1376, 4096], 22 steps of
+        // 128 x 128 tiles: 4 parts 16.4 against 19.5 us unsplit at 128 rows,
+        // 2 parts 25.9 against 20.2 at 512).
         int sk = a.num_sms / k.total_tiles;
         if (sk > nk / 4) sk = nk / 4;
         if (sk > 16) sk = 16;
-        if (sk > 1) {
+        if (sk >= 4 || (sk > 1 && nk >= 32)) {
           k.split_k = sk;
           walk = (nk + sk - 1) / sk;
         }
@@ -170,11 +174,14 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
     // Few parts: the owner's way, which has one hand-over less on its critical
     // path (measured on [128, 4096] x [4096, 1376] with 128 x 128 tiles: 16
     // parts 16.6 against 26.7 us, 8 parts 17.2 against 23.4, 4 parts 23.2
-    // against 25.1, 2 parts 39 against 33).
+    // against 25.1, 2 parts 39 against 33; 64 x 64 tiles in 5 parts 16.2
+    // against 14.9): sliced from eight parts up.
+    // (the 128-accumulator tiles only have the sliced one)
     if (a.split_handover == IRIS_GEMM_HANDOVER_SLICED && k.split_k > pick.cm) return hipErrorInvalidValue;
+    if (a.split_handover == IRIS_GEMM_HANDOVER_OWNER && !pick.split_owner) return hipErrorInvalidValue;
     k.sliced = a.split_handover == IRIS_GEMM_HANDOVER_SLICED  ? 1
                : a.split_handover == IRIS_GEMM_HANDOVER_OWNER ? 0
-                                                              : (k.split_k >= 4 && k.split_k <= pick.cm) ? 1 : 0;
+                                                              : (!pick.split_owner || k.split_k >= 8) ? 1 : 0;
   }
   if (k.stream_k) {
     const int64_t steps = (int64_t)k.total_tiles * nk;

@@ -16,6 +16,7 @@ struct GemmKernelEntry {
   int bk, wm, wn, stages;
   bool dma;    // LDS-DMA loader (needs K-contiguous, 16-byte aligned operands)
   bool splitk;  // the kernel can share a tile's K range with other programs
+  bool split_owner;  // ... and its first part can add the others' partials itself (needed for stream-K runs)
   int threads;
   int lds_bytes;
   GemmKernelFn fn;
@@ -44,7 +45,7 @@ template <class Cfg, int OP>
 constexpr GemmKernelEntry make_entry(const char* name) {
   constexpr int ODT = (OP == OP_STORE32 || OP == OP_ATOMIC32) ? IRIS_DTYPE_F32 : Cfg::DT;
   return GemmKernelEntry{Cfg::DT, OP,      Cfg::CM, Cfg::CN, Cfg::BK,        Cfg::WM,
-                         Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::NT, Cfg::LDS_BYTES,
+                         Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::SPLIT_OWNER, Cfg::NT, Cfg::LDS_BYTES,
                          &gemm_persistent_kernel<Cfg, OP, ODT, false>, split_fn<Cfg, OP, ODT>(), fused_fn<Cfg, OP, ODT>(),
                          name};
 }
@@ -55,9 +56,9 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 // Columns: compute tile CM, CN, BK; waves WM x WN; stages; LDS-DMA loader;
 // whether the tile also has a split-K build (must equal GemmCfg::SPLITK); name.
 #define IRIS_GEMM_VARIANTS(X, DT, OP)                               \
-  X(DT, OP, 256, 256, 64, 2, 4, 2, true, 0, "256x256x64_w2x4_s2")   \
-  X(DT, OP, 256, 128, 64, 2, 2, 2, true, 0, "256x128x64_w2x2_s2")   \
-  X(DT, OP, 128, 256, 64, 1, 4, 2, true, 0, "128x256x64_w1x4_s2")   \
+  X(DT, OP, 256, 256, 64, 2, 4, 2, true, 1, "256x256x64_w2x4_s2")   \
+  X(DT, OP, 256, 128, 64, 2, 2, 2, true, 1, "256x128x64_w2x2_s2")   \
+  X(DT, OP, 128, 256, 64, 1, 4, 2, true, 1, "128x256x64_w1x4_s2")   \
   X(DT, OP, 128, 128, 64, 2, 2, 4, true, 1, "128x128x64_w2x2_s4")   \
   X(DT, OP, 256, 64, 64, 4, 1, 2, true, 1, "256x64x64_w4x1_s2")     \
   X(DT, OP, 64, 64, 64, 2, 2, 4, true, 1, "64x64x64_w2x2_s4")       \

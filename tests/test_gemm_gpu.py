@@ -420,6 +420,9 @@ def split_workspace(shmem, grid, BM, BN):
     (128, 512, 1376, 128, 128, 5),   # 22 K-steps (the last one half empty) in 5 uneven parts
     (200, 72, 776, 256, 64, 4),
     (1, 64, 128, 64, 64, 2),         # one K-step per part
+    (500, 300, 1024, 256, 256, 7),   # 128-accumulator tiles (sliced hand-over only), ragged edges
+    (256, 512, 2048, 256, 128, 16),
+    (128, 500, 640, 128, 256, 3),
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_split_k_all_scatter(shmem, M, N, K, BM, BN, split_k, dtype):
@@ -438,7 +441,10 @@ def test_split_k_all_scatter(shmem, M, N, K, BM, BN, split_k, dtype):
     want = O.shard_gemm(A, B, dtype)
     got = {}
     launch = 0
-    for handover in (ops.HANDOVER_OWNER, ops.HANDOVER_SLICED, ops.HANDOVER_AUTO):
+    ways = (ops.HANDOVER_OWNER, ops.HANDOVER_SLICED, ops.HANDOVER_AUTO)
+    if BM * BN > 128 * 128:
+        ways = (ops.HANDOVER_SLICED, ops.HANDOVER_AUTO)
+    for handover in ways:
         for again in (1, 2):
             launch += 1
             cg.zero_()
@@ -449,7 +455,8 @@ def test_split_k_all_scatter(shmem, M, N, K, BM, BN, split_k, dtype):
             assert flags.cpu().tolist() == [launch] * total
             assert int(locks.abs().max().item()) == 0
         got[handover] = cg.cpu().clone()
-    assert torch.equal(got[ops.HANDOVER_OWNER].view(torch.int16), got[ops.HANDOVER_SLICED].view(torch.int16))
+    if ops.HANDOVER_OWNER in got:
+        assert torch.equal(got[ops.HANDOVER_OWNER].view(torch.int16), got[ops.HANDOVER_SLICED].view(torch.int16))
     assert torch.equal(got[ops.HANDOVER_AUTO].view(torch.int16), got[ops.HANDOVER_SLICED].view(torch.int16))
 
 
@@ -481,9 +488,22 @@ def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
         ops.gemm_launch(*common, split_k=4)                                  # no workspace
     with pytest.raises(ValueError):
         ops.gemm_launch(*common, partials=partials, locks=locks, split_k=16)  # 22 * 16 pairs > 256 programs
+    # the 128-accumulator tiles split too, with the sliced hand-over only
+    big = shmem.zeros((256, 256 * 256), dtype=torch.float32)
     with pytest.raises(ValueError):
         ops.gemm_launch(a2, b2, None, cg2, flags2, None, 0, 1, 256, 256, 256, 64, 4, ops.EPI_ALL_SCATTER,
-                        partials=shmem.zeros((256, 256 * 256), dtype=torch.float32), locks=locks, split_k=2)
+                        partials=big, locks=locks, split_k=2, split_handover=ops.HANDOVER_OWNER)
+    with pytest.raises(ValueError):  # and never stream-K
+        ops.gemm_launch(a2, b2, None, cg2, flags2, None, 0, 1, 256, 256, 256, 64, 4, ops.EPI_ALL_SCATTER,
+                        partials=big, locks=locks, split_k=ops.SPLIT_STREAM_K)
+    for sk in (2, 8):
+        cg2.zero_()
+        flags2.zero_()
+        ops.gemm_launch(a2, b2, None, cg2, flags2, None, 0, 1, 256, 256, 256, 64, 4, ops.EPI_ALL_SCATTER,
+                        partials=big, locks=locks, split_k=sk)
+        torch.cuda.synchronize()
+        check_close(cg2, O.shard_gemm(A2, B2, dtype), f"256 x 256 tiles in {sk} parts")
+        assert flags2.cpu().tolist()[:16] == [1] * 16 and int(locks.abs().max().item()) == 0
 
 
 STREAM_K_CASES = [
@@ -540,7 +560,7 @@ def test_stream_k_is_chosen_when_the_last_round_of_tiles_is_thin(shmem):
     assert choice(88, 128, 128) == 1                         # one tile each
     assert choice(44, 128, 128) == 1                         # two rounds, both full
     assert choice(256, 128, 128, split_k=1) == 1
-    assert choice(256, 256, 256) == 1                        # a tile whose kernel has no split build
+    assert choice(256, 256, 256) == 1                        # the workspace's slots are too small for this tile
     ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 256, 128, 128, 64, 4, ops.EPI_ALL_SCATTER, partials=partials,
                     locks=locks)
     torch.cuda.synchronize()
