@@ -51,6 +51,61 @@ __host__ __device__ inline TileCoord tile_map(int tile_id, int num_pid_m, int nu
   return t;
 }
 
+// Division of a launch's small integers (tile and item indices) by a divisor
+// that is fixed for the launch, as a multiply-high: with m = ceil(2^32 / d),
+// floor(n m / 2^32) = floor(n / d) for every n with n d < 2^32 (the error term
+// n (m d - 2^32) / (d 2^32) stays below 1 / d).  The launcher fills `m` when
+// every dividend of the launch obeys that bound and leaves 0 otherwise; the
+// kernels then fall back to the hardware-less division sequence.  A tile
+// switch of the persistent kernels decodes two tiles with five divisions each,
+// in every wave: ~200 scalar instructions apiece as division sequences, a
+// dozen this way.
+struct FastDiv {
+  uint32_t d, m;
+};
+__host__ __device__ inline FastDiv make_fast_div(uint32_t d, uint64_t max_dividend) {
+  FastDiv f{d ? d : 1u, 0u};
+  if (f.d > 1 && max_dividend * f.d < ((uint64_t)1 << 32)) f.m = (uint32_t)((((uint64_t)1 << 32) + f.d - 1) / f.d);
+  return f;
+}
+__host__ __device__ inline uint32_t fast_div(uint32_t n, const FastDiv& f) {
+  if (f.d == 1) return n;
+  if (f.m) return (uint32_t)(((uint64_t)n * f.m) >> 32);
+  return n / f.d;
+}
+
+// The divisors of a launch's tile decode.
+struct TileDivs {
+  FastDiv in_group;  // G * num_pid_n: tiles per group of G tile rows
+  FastDiv group;     // G: rows of a full group
+  FastDiv tail;      // num_pid_m % G: rows of the last, short group (1 when there is none)
+};
+__host__ __device__ inline TileDivs make_tile_divs(int num_pid_m, int num_pid_n, int G) {
+  const uint64_t total = (uint64_t)num_pid_m * num_pid_n + 1;
+  TileDivs t;
+  t.in_group = make_fast_div((uint32_t)(G * num_pid_n), total);
+  t.group = make_fast_div((uint32_t)G, total);
+  t.tail = make_fast_div((uint32_t)(num_pid_m % G ? num_pid_m % G : 1), total);
+  return t;
+}
+// tile_map with the launch's precomputed divisors: the same arithmetic.
+__host__ __device__ inline TileCoord tile_map_fast(int tile_id, int num_pid_m, int num_pid_n, int G,
+                                                   const TileDivs& dv) {
+  const int group_id = (int)fast_div((uint32_t)tile_id, dv.in_group);
+  const int first_pid_m = group_id * G;
+  const int rem = num_pid_m - first_pid_m;
+  const int in_group = tile_id - group_id * (G * num_pid_n);
+  TileCoord t;
+  if (rem < G) {  // the last group, num_pid_m % G rows
+    t.pid_n = (int)fast_div((uint32_t)in_group, dv.tail);
+    t.pid_m = first_pid_m + in_group - t.pid_n * rem;
+  } else {
+    t.pid_n = (int)fast_div((uint32_t)in_group, dv.group);
+    t.pid_m = first_pid_m + in_group - t.pid_n * G;
+  }
+  return t;
+}
+
 // (pid_m, pid_n) -> tile_id: the inverse of tile_map.
 __host__ __device__ inline int tile_id_of(int pid_m, int pid_n, int num_pid_m, int num_pid_n, int G) {
   const int group_id = pid_m / G;

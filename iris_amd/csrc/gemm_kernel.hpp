@@ -59,6 +59,10 @@ struct GemmKArgs {
   int xcd_per;
   int num_pid_m, num_pid_n, total_tiles;
   int sub_m, sub_n;  // compute tiles per logical tile
+  // the launch's divisors, for the tile decode (see FastDiv)
+  TileDivs tile_divs;
+  FastDiv div_subs, div_sub_n;  // sub_m * sub_n, sub_n
+  FastDiv div_split, div_nk;    // split_k; K-steps of a tile (stream-K runs)
   int dest_all;      // write `out` on every rank's heap (else on this rank only)
   int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
   int sys;           // flag atomics at system scope (else agent)
@@ -187,7 +191,7 @@ __host__ __device__ inline StreamRun stream_run(const GemmKArgs& p, int pid, int
   StreamRun r;
   const int g0 = pid * p.split_q + (pid < p.split_r ? pid : p.split_r);
   r.g1 = g0 + stream_len(p, pid);
-  r.tile0 = nk > 0 ? g0 / nk : 0;
+  r.tile0 = nk > 0 ? (int)fast_div((uint32_t)g0, p.div_nk) : 0;
   r.k0 = g0 - r.tile0 * nk;
   return r;
 }
@@ -206,7 +210,7 @@ __host__ __device__ inline int stream_parts(const GemmKArgs& p, int pid, int k_e
 // pid is part pid % split_k of tile pid / split_k (one item per program).
 __device__ inline StreamRun split_run(const GemmKArgs& p, int pid, int nk) {
   StreamRun r;
-  r.tile0 = (int)((unsigned)pid / (unsigned)p.split_k);
+  r.tile0 = (int)fast_div((uint32_t)pid, p.div_split);
   const int part = pid - r.tile0 * p.split_k;
   r.k0 = part * p.split_q + min(part, p.split_r);
   r.g1 = r.tile0 * nk + r.k0 + (r.tile0 < p.total_tiles ? p.split_q + (part < p.split_r ? 1 : 0) : 0);
@@ -237,7 +241,7 @@ __device__ inline Item decode_item(const GemmKArgs& p, const StreamRun& sr, int 
     // one compute tile per logical tile; the program's run touches tiles
     // tile0, tile0 + 1, ...
     it.tile_id = sr.tile0 + item;
-    const TileCoord tc = tile_map(it.tile_id, p.num_pid_m, p.num_pid_n, p.G);
+    const TileCoord tc = tile_map_fast(it.tile_id, p.num_pid_m, p.num_pid_n, p.G, p.tile_divs);
     it.lm0 = it.m0 = tc.pid_m * p.BM;
     it.ln0 = it.n0 = tc.pid_n * p.BN;
     it.m_end = min(p.M, it.lm0 + p.BM);
@@ -245,13 +249,13 @@ __device__ inline Item decode_item(const GemmKArgs& p, const StreamRun& sr, int 
     it.first_sub = it.last_sub = true;
     return it;
   }
-  const int ti = item / subs;
+  const int ti = (int)fast_div((uint32_t)item, p.div_subs);
   const int s = item - ti * subs;
   it.tile_id = pid + ti * p.num_sms;
-  const TileCoord tc = tile_map(it.tile_id, p.num_pid_m, p.num_pid_n, p.G);
+  const TileCoord tc = tile_map_fast(it.tile_id, p.num_pid_m, p.num_pid_n, p.G, p.tile_divs);
   it.lm0 = tc.pid_m * p.BM;
   it.ln0 = tc.pid_n * p.BN;
-  const int sm = s / p.sub_n, sn = s - sm * p.sub_n;
+  const int sm = (int)fast_div((uint32_t)s, p.div_sub_n), sn = s - sm * p.sub_n;
   it.m0 = it.lm0 + sm * Cfg::CM;
   it.n0 = it.ln0 + sn * Cfg::CN;
   it.m_end = min(p.M, it.lm0 + p.BM);
@@ -1052,7 +1056,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       if (p.sliced) {
         // split-K proper: program pid is part pid % split_k of tile pid / split_k
         const int parts = p.split_k;
-        const int slot0 = __builtin_amdgcn_readfirstlane((int)((unsigned)pid / (unsigned)parts) * parts);
+        const int slot0 = __builtin_amdgcn_readfirstlane((int)fast_div((uint32_t)pid, p.div_split) * parts);
         const int part = pid - slot0;
         IRIS_LDS int* okslot = (IRIS_LDS int*)(lds + Cfg::S * Cfg::STAGE);  // wave 0's scratch, idle here
         {

@@ -359,6 +359,16 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   plan->entry = pick;
 
   const hipError_t err = plan_split(a, *pick, plan->in_program != 0, &k);
+  {
+    // the launch's divisors as multiply-high constants
+    const int nk = (a.K + pick->bk - 1) / pick->bk;
+    const uint64_t items = (uint64_t)k.total_tiles * k.sub_m * k.sub_n + 1;
+    k.tile_divs = make_tile_divs(k.num_pid_m, k.num_pid_n, k.G);
+    k.div_subs = make_fast_div((uint32_t)(k.sub_m * k.sub_n), items);
+    k.div_sub_n = make_fast_div((uint32_t)k.sub_n, items);
+    k.div_split = make_fast_div((uint32_t)k.split_k, (uint64_t)a.num_sms + 1);
+    k.div_nk = make_fast_div((uint32_t)(nk > 0 ? nk : 1), (uint64_t)k.total_tiles * (nk > 0 ? nk : 1) + 1);
+  }
   // (under stream-K every program has a run: the reference's XCD remap stays)
   if (err != hipSuccess || k.stream_k) return err;
   // Fewer (tile, part) items than programs: deal them to the XCDs evenly, in
@@ -621,6 +631,7 @@ extern "C" int iris_stream_k_schedule_host(int32_t total_tiles, int32_t k_steps,
   k.split_q = (int)(steps / num_programs);
   k.split_r = (int)(steps % num_programs);
   if (k.split_q < 1) return hipErrorInvalidValue;  // the kernel is never launched with empty runs
+  k.div_nk = make_fast_div((uint32_t)k_steps, (uint64_t)steps + 1);
   const StreamRun sr = stream_run(k, pid, k_steps);
   const int n = stream_items(sr, k_steps);
   *n_items = n;

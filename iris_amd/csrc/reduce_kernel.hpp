@@ -352,13 +352,13 @@ __global__ __launch_bounds__(256) void signal_tiles_kernel(int32_t* flags, const
 // (pid_m, pid_n, owning program, position in that program's tile list).
 // Program p of a grid of num_sms visits xcd_remap(p), +num_sms, ...
 __global__ __launch_bounds__(256) void tile_schedule_kernel(int32_t* out, int num_pid_m, int num_pid_n, int G,
-                                                            int num_sms, int num_xcds) {
+                                                            int num_sms, int num_xcds, TileDivs divs) {
   const int prog = blockIdx.x * 256 + threadIdx.x;
   if (prog >= num_sms) return;
   const int total = num_pid_m * num_pid_n;
   int pos = 0;
   for (int t = xcd_remap(prog, num_sms, num_xcds); t < total; t += num_sms, ++pos) {
-    const TileCoord tc = tile_map(t, num_pid_m, num_pid_n, G);
+    const TileCoord tc = tile_map_fast(t, num_pid_m, num_pid_n, G, divs);  // as the GEMM kernels decode a tile
     out[4 * t + 0] = tc.pid_m;
     out[4 * t + 1] = tc.pid_n;
     out[4 * t + 2] = prog;

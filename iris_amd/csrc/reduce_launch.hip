@@ -186,14 +186,16 @@ extern "C" int iris_tile_schedule_launch(int32_t* out, int32_t M, int32_t N, int
     return hipErrorInvalidValue;
   const int npm = (M + block_m - 1) / block_m, npn = (N + block_n - 1) / block_n;
   hipLaunchKernelGGL(tile_schedule_kernel, dim3((num_sms + 255) / 256), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), out, npm, npn, group_size_m, num_sms, num_xcds);
+                     static_cast<hipStream_t>(stream), out, npm, npn, group_size_m, num_sms, num_xcds,
+                     make_tile_divs(npm, npn, group_size_m));
   return hipGetLastError();
 }
 
 extern "C" void iris_tile_map_host(int32_t tile_id, int32_t M, int32_t N, int32_t block_m, int32_t block_n,
                                    int32_t group_size_m, int32_t* pid_m, int32_t* pid_n) {
-  const TileCoord tc =
-      tile_map(tile_id, (M + block_m - 1) / block_m, (N + block_n - 1) / block_n, group_size_m);
+  // (the GEMM kernels' arithmetic: multiply-high divisions by the launch's divisors)
+  const int npm = (M + block_m - 1) / block_m, npn = (N + block_n - 1) / block_n;
+  const TileCoord tc = tile_map_fast(tile_id, npm, npn, group_size_m, make_tile_divs(npm, npn, group_size_m));
   *pid_m = tc.pid_m;
   *pid_n = tc.pid_n;
 }

@@ -103,7 +103,8 @@ def test_host_build_of_the_kernel_tile_map_is_bit_exact():
 
     for M, N, BM, BN, G in [(8192, 8192, 256, 256, 4), (8192, 8192, 256, 256, 6), (4096, 4096, 256, 256, 6),
                             (2048, 1376, 256, 64, 4), (1, 1376, 256, 256, 8), (1000, 999, 64, 64, 5),
-                            (8192, 4608, 256, 64, 4), (768, 512, 256, 128, 6)]:
+                            (8192, 4608, 256, 64, 4), (768, 512, 256, 128, 6), (16384, 16384, 64, 64, 7),
+                            (8192, 200, 32, 200, 3), (40, 40, 8, 8, 1), (256, 100000, 256, 16, 2)]:
         total = O.cdiv(M, BM) * O.cdiv(N, BN)
         want = O.tile_map_all(M, N, BM, BN, G)
         got = [ops.tile_map_host(t, M, N, BM, BN, G) for t in range(total)]
