@@ -166,7 +166,7 @@ typedef struct iris_gemm_args {
    * the hand-over.  Results differ from the unsplit ones only in fp32
    * summation order. */
   float* partials;      /* [num_sms][partials_slot_elems] fp32, or NULL           */
-  int32_t* locks;       /* int32[num_sms], or NULL                                */
+  int32_t* locks;       /* int32[num_sms], or NULL (a tile in n parts uses the n words of its programs) */
   int64_t partials_slot_elems; /* >= block_m * block_n                            */
   int32_t split_k;      /* 0 = let the launcher decide, 1 = never, n > 1 = force n, IRIS_GEMM_SPLIT_STREAM_K */
   /* How the parts of a split tile meet (split-K proper; stream-K runs always
