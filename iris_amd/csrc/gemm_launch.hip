@@ -375,6 +375,18 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   // consecutive runs, instead of filling the first XCDs and idling the rest.
   const int64_t work = (int64_t)k.total_tiles * k.split_k;
   if (a.num_xcds > 1 && work < a.num_sms) k.xcd_per = (int)((work + a.num_xcds - 1) / a.num_xcds);
+  // A tile whose stages take at most half a CU's LDS runs one wave per SIMD
+  // and has every instruction of a K-step on its critical path.  A launch
+  // that owns the whole device (one program per CU or more) and has at least
+  // two such tiles per program is given two programs per CU, each other's
+  // cover: which program computes which tile is not observable, the tiles'
+  // flags are.  (64 x 64 tiles, 256 -> 512 programs: [512,1376] x [1376,4096]
+  // 25.0 -> 17.8 us, [2048,4096] x [4096,1376] 80 -> 65 us.)
+  const int64_t items = (int64_t)k.total_tiles * k.sub_m * k.sub_n;
+  if (!plan->in_program && k.split_k == 1 && pick->lds_bytes * 2 <= 160 * 1024 && a.num_sms >= current_cu_count() &&
+      a.num_sms <= 2 * current_cu_count() && items >= 2 * (int64_t)a.num_sms && !a.mm_begin_timestamp &&
+      !a.mm_end_timestamp)
+    k.num_sms = 2 * a.num_sms;
   return hipSuccess;
 }
 
@@ -617,7 +629,10 @@ extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t
   hipError_t err = make_plan(*args, &plan);
   if (err != hipSuccess) return err;
   std::snprintf(buf, len, "%s%s", plan.skinny ? "few_rows_16xN" : plan.entry ? plan.entry->name : "",
-                plan.entry && plan.k.stream_k ? "+stream_k" : plan.entry && plan.in_program ? "+reduce" : "");
+                plan.entry && plan.k.stream_k                   ? "+stream_k"
+                : plan.entry && plan.in_program                 ? "+reduce"
+                : plan.entry && plan.k.num_sms > args->num_sms ? "+two_per_cu"
+                                                                : "");
   return hipSuccess;
 }
 

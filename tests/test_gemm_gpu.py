@@ -408,6 +408,28 @@ def test_launcher_rejects_what_the_kernels_do_not_take(shmem):
                         notify=False)
 
 
+def test_small_tiles_get_two_programs_per_cu_when_the_launch_owns_the_device(shmem):
+    """64 x 64 tiles take less than half a CU's LDS: a launch with one program
+    per CU and two tiles or more per program runs two programs per CU.  Which
+    program computes a tile is not observable: values and flags are checked."""
+    dtype = torch.bfloat16
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    M, N, K, BM, BN = 2048, 1024, 320, 64, 64
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    args = (a, b, None, cg, flags, None, 0, 1, cus, BM, BN, 64, 4, ops.EPI_ALL_SCATTER)
+    assert total >= 2 * cus and ops.gemm_plan_name(*args, num_xcds=8).endswith("+two_per_cu")
+    assert not ops.gemm_plan_name(a, b, None, cg, flags, None, 0, 1, cus // 2, BM, BN, 64, 4, ops.EPI_ALL_SCATTER,
+                                  num_xcds=8).endswith("+two_per_cu")  # half the device: the grid is the caller's
+    ops.gemm_launch(*args, num_xcds=8)
+    torch.cuda.synchronize()
+    check_close(cg, O.shard_gemm(A, B, dtype))
+    assert flags.cpu().tolist() == [1] * total
+
+
 # --------------------------------------------------------------------------- split-K
 def split_workspace(shmem, grid, BM, BN):
     return (shmem.zeros((grid, BM * BN), dtype=torch.float32), shmem.zeros((grid,), dtype=torch.int32))
