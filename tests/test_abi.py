@@ -111,6 +111,26 @@ def test_host_build_of_the_kernel_tile_map_is_bit_exact():
         assert got == [tuple(r) for r in want.tolist()]
 
 
+def test_host_build_of_the_tile_map_beyond_the_multiply_high_bound():
+    """Tile grids too large for the multiply-high constants (tile id times
+    divisor no longer fits 32 bits) make the kernels divide instead: sampled
+    tile ids of such grids, and of grids just inside the bound, against the
+    oracle."""
+    import random
+
+    from iris_amd import ops
+    from oracle import iris_oracle as O
+
+    rng = random.Random(7)
+    for M, N, BM, BN, G in [(40000, 40000, 1, 1, 8), (46000, 46000, 1, 1, 3), (3000, 90000, 1, 1, 7),
+                            (46340, 46340, 1, 1, 1), (1 << 20, 2000, 512, 1, 5)]:
+        total = O.cdiv(M, BM) * O.cdiv(N, BN)
+        assert total < (1 << 31)
+        ids = [0, 1, total - 1, total - 2] + [rng.randrange(total) for _ in range(400)]
+        for t in ids:
+            assert ops.tile_map_host(t, M, N, BM, BN, G) == O.tile_map(t, M, N, BM, BN, G), (t, M, N, G)
+
+
 def test_host_build_of_the_stream_k_schedule_partitions_the_k_steps():
     """The kernels' stream-K run arithmetic, compiled for the host: the runs
     cut the launch's K-steps without gap or overlap, differ by at most one
