@@ -233,6 +233,21 @@ def context_figures(a, b, c_global, flops, gemm_on):
         ms = steady_ms(lambda: ops.mfma_probe(operands, sink, iters, groups), n=100)
         out[f"mfma_sustained[{name}]"] = {"what": "register-only v_mfma_f32_16x16x32_bf16 loop, 8 waves per CU",
                                            "tflops": round(fl / (ms * 1e-3) / 1e12, 1)}
+        # what the output stores of the headline launch cost next to the matrix cores, and whether spreading
+        # them helps: 4 tiles a CU of register-only MFMAs (a 256x256x1024 tile's worth each) with 128 KiB of
+        # write-through stores a tile, all at once / one KiB a wave and K-step / none (iris_store_probe_launch)
+        tiles = 4
+        region = torch.empty(tiles * groups * 131072, dtype=torch.uint8, device="cuda")
+        t = {}
+        for label, chunk in (("none", 0), ("tile_at_once", 16), ("one_store_per_k_step", 1)):
+            t[label] = steady_ms(lambda: ops.store_probe(operands, sink, region, tiles, chunk, groups), n=100) * 1e3
+        out[f"store_cost[{name}]"] = {
+            "what": "register-only MFMAs of 4 tiles a CU + 128 MiB of write-through stores (16 one-KiB stores a wave "
+                    "and tile), us per launch",
+            "mfma_only_us": round(t["none"], 1),
+            "tile_at_once_extra_us": round(t["tile_at_once"] - t["none"], 1),
+            "one_store_per_k_step_extra_us": round(t["one_store_per_k_step"] - t["none"], 1)}
+        del region
     return out
 
 

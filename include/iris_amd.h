@@ -306,6 +306,22 @@ int iris_mfma_probe_launch(const void* operands, float* sink, int32_t ab_dtype, 
                            void* stream);
 
 /*
+ * Measurement aid; no counterpart in the reference.  What a tile's worth of
+ * output stores costs next to the matrix cores, by how the stores are spread:
+ * each of `num_groups` workgroups of 8 waves runs `tiles` tiles, a tile being
+ * 16 K-steps of 64 register-only bf16 MFMAs a wave (a 256 x 256 x 1024 tile's
+ * worth) and 16 one-KiB stores a wave (128 KiB a group) to a region of its own
+ * in `out` (`out_bytes` >= num_groups * 128 KiB, 16-byte aligned; tile t goes
+ * to offset t * num_groups * 128 KiB modulo what fits).  `chunk` stores go out
+ * back to back every `chunk` K-steps: 16 = a whole tile at once, 4, 1 = one a
+ * K-step, 0 = none.  `write_through`: sc1 stores (else plain); `lockstep`: the
+ * waves of a group meet at a barrier after every K-step.  `operands` and
+ * `sink` as for iris_mfma_probe_launch.
+ */
+int iris_store_probe_launch(const void* operands, float* sink, void* out, uint64_t out_bytes, int32_t tiles,
+                            int32_t chunk, int32_t write_through, int32_t lockstep, int32_t num_groups, void* stream);
+
+/*
  * Device-side remote access (include/iris_device.hpp, the HIP counterpart of
  * iris/iris.py:317-521) exercised the way the reference's unit tests exercise
  * the Triton functions: one workgroup, lane i < block_size owns element i of

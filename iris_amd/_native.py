@@ -146,6 +146,7 @@ SIGNATURES = {
     "iris_stream_k_schedule_host": (_I, [ctypes.c_int32] * 4 + [ctypes.POINTER(ctypes.c_int32), ctypes.c_int32,
                                          ctypes.POINTER(ctypes.c_int32)]),
     "iris_mfma_probe_launch": (_I, [_P, _P, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P]),
+    "iris_store_probe_launch": (_I, [_P, _P, _P, ctypes.c_uint64] + [ctypes.c_int32] * 5 + [_P]),
     "iris_rma_selftest_launch": (_I, [ctypes.c_int32] * 4 + [_P, _P, _P] + [ctypes.c_int32] * 3 + [_P]),
     "iris_p2p_bench_launch": (_I, [ctypes.c_int32] * 2 + [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 3
                               + [_P, ctypes.c_int32, _P]),

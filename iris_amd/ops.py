@@ -41,6 +41,7 @@ __all__ = [
     "gemm_plan_name",
     "stream_k_schedule_host",
     "gemm_variant_name",
+    "store_probe",
     "one_shot_reduce",
     "signal_tiles",
     "tile_schedule",
@@ -427,6 +428,28 @@ def mfma_probe(operands, sink, iters, num_groups):
     _native.hip_try(_native.lib().iris_mfma_probe_launch(_ptr(operands), _ptr(sink), _DTYPES[operands.dtype], iters,
                                                          num_groups, ctypes.c_void_p(stream)))
     return num_groups * 8 * iters * 16 * 16384
+
+
+def store_probe(operands, sink, out, tiles, chunk, num_groups, *, write_through=True, lockstep=True):
+    """Launch the store probe (a measurement aid): ``tiles`` tiles per group of
+    8 waves, each 16 K-steps of register-only MFMAs and 128 KiB of stores to
+    ``out``, ``chunk`` one-KiB stores a wave back to back every ``chunk``
+    K-steps (16, 4, 1, or 0 for none).  Returns the bytes stored per launch."""
+    if operands.dtype != torch.bfloat16 or operands.numel() * 2 < 65536 or not operands.is_contiguous():
+        raise ValueError("operands: at least 64 KiB of contiguous bf16")
+    if sink.dtype != torch.float32 or sink.numel() < num_groups * 512:
+        raise ValueError("sink: at least num_groups * 512 floats")
+    out_bytes = out.numel() * out.element_size()
+    if not out.is_contiguous() or out_bytes < num_groups * 131072:
+        raise ValueError("out: contiguous, at least 128 KiB per group")
+    stream = torch.cuda.current_stream(operands.device).cuda_stream
+    err = _native.lib().iris_store_probe_launch(_ptr(operands), _ptr(sink), _ptr(out), out_bytes, tiles, chunk,
+                                                1 if write_through else 0, 1 if lockstep else 0, num_groups,
+                                                ctypes.c_void_p(stream))
+    if err == _native.HIP_ERROR_INVALID_VALUE:
+        raise ValueError("iris_store_probe_launch rejected the arguments")
+    _native.hip_try(err)
+    return 0 if chunk == 0 else tiles * num_groups * 131072
 
 
 def rma_selftest(op, data, results, heap_bases, rank, num_ranks, block_size, *, sem="acq_rel", scope="sys"):

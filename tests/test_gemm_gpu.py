@@ -430,6 +430,32 @@ def test_small_tiles_get_two_programs_per_cu_when_the_launch_owns_the_device(shm
     assert flags.cpu().tolist() == [1] * total
 
 
+def test_store_probe_writes_every_groups_region(shmem):
+    """The store probe (a measurement aid): every wave writes its 16 KiB of
+    every tile, whatever the spreading, and nothing outside."""
+    groups, tiles = 8, 3
+    operands = torch.ones(32768, dtype=torch.bfloat16, device="cuda")
+    sink = torch.zeros(groups * 512, dtype=torch.float32, device="cuda")
+    for chunk in (16, 4, 1):
+        for wt in (True, False):
+            out = torch.full((tiles * groups * 131072 + 4096,), 0x5A, dtype=torch.uint8, device="cuda")
+            assert ops.store_probe(operands, sink, out[:-4096], tiles, chunk, groups, write_through=wt) == tiles * groups * 131072
+            torch.cuda.synchronize()
+            body = out[:-4096].view(torch.float32)
+            # accumulators of ones x ones products: whole numbers, never the fill pattern
+            assert bool((body == body.round()).all()) and bool((body > 0).any())
+            assert not bool((out[:-4096] == 0x5A).view(-1, 16).all(dim=1).any()), "a 16-byte unit was not written"
+            assert bool((out[-4096:] == 0x5A).all())
+    out = torch.full((groups * 131072,), 0x5A, dtype=torch.uint8, device="cuda")
+    assert ops.store_probe(operands, sink, out, tiles, 0, groups) == 0
+    torch.cuda.synchronize()
+    assert bool((out == 0x5A).all()) and bool(torch.isfinite(sink).all())
+    with pytest.raises(ValueError):
+        ops.store_probe(operands, sink, out[:1000], tiles, 16, groups)
+    with pytest.raises(ValueError):
+        ops.store_probe(operands, sink, out, tiles, 3, groups)
+
+
 # --------------------------------------------------------------------------- split-K
 def split_workspace(shmem, grid, BM, BN):
     return (shmem.zeros((grid, BM * BN), dtype=torch.float32), shmem.zeros((grid,), dtype=torch.int32))
