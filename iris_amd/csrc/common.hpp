@@ -318,13 +318,14 @@ __device__ inline bool wait_tile_flag(IRIS_GLOBAL int32_t* flag, int ws, bool sy
 
 // Bounded wait until a tile's flag has reached `need`, without consuming it.
 // Returns whether it has; a wait that gives up records IRIS_STATUS_SPIN_TIMEOUT.
+// `mask` selects the bits of the flag that count.
 __device__ inline bool wait_tile_ready(IRIS_GLOBAL int32_t* flag, int need, bool sys, uint64_t timeout,
-                                       uint32_t* status) {
+                                       uint32_t* status, int mask = -1) {
   const uint64_t t0 = wall_clock64();
   for (;;) {
     const int v = sys ? __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)
                       : __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (v >= need) return true;
+    if ((v & mask) >= need) return true;
     if (wall_clock64() - t0 > timeout) {
       if (status) atomicMax(status, (uint32_t)IRIS_STATUS_SPIN_TIMEOUT);
       return false;

@@ -31,7 +31,15 @@ struct ReduceKArgs {
   int band_rows, band_vecs, band_chunks, band_items;
   // tile kernel: fetch the ranks' heap bases with vector loads (see there)
   int pace;
+  // row-band kernel: the group that finishes last takes the consumed flags
+  // back to 0 (else the launcher enqueues reset_consumed_flags_kernel)
+  int reset_in_kernel;
 };
+
+// The row-band kernel counts its finished groups in the upper half of the
+// first tile's flag (a producer's +1 only ever touches the lower half), so a
+// flag's value is its lower half.
+constexpr int FLAG_COUNT_SHIFT = 16, FLAG_VALUE_MASK = 0xFFFF;
 
 // Block-wide wait for one tile's flag.  One lane polls; the outcome is
 // broadcast through LDS and every wave then acquires.
@@ -156,8 +164,10 @@ __global__ __launch_bounds__(256) void reduce_tiles_vec_kernel(const ReduceKArgs
 // Flags: the band crosses every tile of its tile row, so the group waits for
 // all of them (one lane per tile) without consuming them; a tile that does
 // not arrive within the timeout only masks its own columns.  The flags that
-// reached ws-1 are reset to 0 by reset_consumed_flags_kernel, which the
-// launcher enqueues behind this kernel.  The sum is in rank order 0..ws-1.
+// reached ws-1 are reset to 0 by the group that finishes last (the groups
+// count themselves on the upper half of the first flag), or, for grids too
+// large for that count, by reset_consumed_flags_kernel, which the launcher
+// then enqueues behind this kernel.  The sum is in rank order 0..ws-1.
 template <int IN_DT, int OUT_DT, int LAUX, int WS>
 __global__ __launch_bounds__(256) void reduce_rows_kernel(const ReduceKArgs p) {
   constexpr int IES = Vec<IN_DT>::ES, VE = Vec<IN_DT>::N, OES = Vec<OUT_DT>::ES;
@@ -203,7 +213,10 @@ __global__ __launch_bounds__(256) void reduce_rows_kernel(const ReduceKArgs p) {
       int ok = 1;
       if (tid < ntn) {
         const int t = tile_id_of(row0 / p.BM, tn0 + tid, p.num_pid_m, p.num_pid_n, p.G);
-        ok = wait_tile_ready((IRIS_GLOBAL int32_t*)(p.flags + t), p.ws - 1, p.sys != 0, p.timeout, p.status) ? 1 : 0;
+        ok = wait_tile_ready((IRIS_GLOBAL int32_t*)(p.flags + t), p.ws - 1, p.sys != 0, p.timeout, p.status,
+                             FLAG_VALUE_MASK)
+                 ? 1
+                 : 0;
         ready[tid] = ok;
       }
       all = __syncthreads_and(ok) != 0;
@@ -279,6 +292,34 @@ __global__ __launch_bounds__(256) void reduce_rows_kernel(const ReduceKArgs p) {
 #pragma unroll
     for (int k = 0; k < K; ++k) store_vec<OUT_DT, VE, SAUX>(out_rs, ooff[k], acc[k]);
     if (wait) __syncthreads();  // `ready` is rewritten for the next item
+  }
+  if (wait && p.reset_in_kernel) {
+    // This group is past all its waits.  Groups count themselves on the upper
+    // half of flags[0]; the one that counts last knows that nobody polls any
+    // more and takes every flag that reached ws-1 back to 0, which is what the
+    // consumer's CAS(ws-1 -> 0) leaves (gemm_one_shot_all_reduce.py:228-234).
+    // The count comes off with one atomic per flag, so a +1 of the next round
+    // that lands meanwhile is kept.
+    if (tid == 0) {
+      // (at the flags' scope, like the producers' increments of the same word)
+      const int before = p.sys ? __hip_atomic_fetch_add((IRIS_GLOBAL int32_t*)p.flags, 1 << FLAG_COUNT_SHIFT,
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)
+                               : __hip_atomic_fetch_add((IRIS_GLOBAL int32_t*)p.flags, 1 << FLAG_COUNT_SHIFT,
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      ready[0] = (before >> FLAG_COUNT_SHIFT) == (int)gridDim.x - 1 ? 1 : 0;
+    }
+    __syncthreads();
+    if (ready[0]) {
+      const int consumed = p.ws - 1;
+      for (int t = tid; t < p.total_tiles; t += 256) {
+        IRIS_GLOBAL int32_t* f = (IRIS_GLOBAL int32_t*)(p.flags + t);
+        const int v = p.sys ? __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)
+                            : __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int take = (v & FLAG_VALUE_MASK) >= consumed ? consumed : 0;
+        if (t == 0) take += (int)gridDim.x << FLAG_COUNT_SHIFT;  // the groups' count, too
+        if (take) flag_add_relaxed(f, -take, p.sys != 0);
+      }
+    }
   }
 }
 

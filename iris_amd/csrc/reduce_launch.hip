@@ -147,9 +147,11 @@ extern "C" int iris_one_shot_reduce_launch(const iris_reduce_args* a, void* stre
     grid = a->num_sms > 0 ? a->num_sms : 2 * current_cu_count();
     if (grid > k.band_items) grid = k.band_items;
   }
+  // (the groups' count shares a 32-bit flag with a value below 2^16)
+  k.reset_in_kernel = (rows && k.wait_flags && k.ws > 1 && grid < (1 << 15) && k.ws <= (1 << 15)) ? 1 : 0;
   hipLaunchKernelGGL(fn, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), k);
   hipError_t err = hipGetLastError();
-  if (err == hipSuccess && rows && k.wait_flags && k.ws > 1) {
+  if (err == hipSuccess && rows && k.wait_flags && k.ws > 1 && !k.reset_in_kernel) {
     hipLaunchKernelGGL(reset_consumed_flags_kernel, dim3((k.total_tiles + 255) / 256), dim3(256), 0,
                        static_cast<hipStream_t>(stream), k.flags, k.ws - 1, k.total_tiles);
     err = hipGetLastError();
