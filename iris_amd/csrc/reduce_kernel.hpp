@@ -324,11 +324,11 @@ __global__ __launch_bounds__(256) void reduce_rows_kernel(const ReduceKArgs p) {
 }
 
 // Flags that the row-band kernel has consumed (value ws-1) back to 0, as the
-// consumer's CAS(ws-1 -> 0) leaves them (gemm_one_shot_all_reduce.py:228-234).
-// The count is taken off with one atomic: a +1 of the next round that lands
-// on the flag meanwhile is kept.  (Counting the consumers on the flags inside
-// the reduce kernel instead was measured: atomics that return a value to a few
-// hot addresses cost the row walk 12-50 % of its bandwidth.)
+// consumer's CAS(ws-1 -> 0) leaves them (gemm_one_shot_all_reduce.py:228-234):
+// the stand-in, as a kernel behind the reduce, for the reset by the group
+// that finishes last, when the grid is too large for that group count.  The
+// count is taken off with one atomic: a +1 of the next round that lands on
+// the flag meanwhile is kept.
 __global__ __launch_bounds__(256) void reset_consumed_flags_kernel(int32_t* flags, int consumed, int total) {
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= total) return;
