@@ -553,9 +553,6 @@ def main():
         },
     }
 
-    if not args.no_context:
-        result["context"] = context_figures(a, b, c_global, flops, gemm_on)
-
     if not args.no_coldcache:
         # the reference's own timing protocol (iris/util.py:62-104): every repetition starts behind a 256 MiB
         # cache flush and a device synchronise, one event pair per launch
@@ -614,6 +611,31 @@ def main():
                          "frac": round(gbps / PEAK_HBM_GBPS, 4),
                          "traffic": REDUCE_TRAFFIC_BYTES if args.reduce_variant == 0 else None},
         }
+        if not args.no_context:
+            # the same launch with other numbers of groups (the default is two per CU): the rate follows the
+            # groups a CU hosts, not the bytes it requests; 10 launches each, flags armed beforehand as above
+            sweep = {}
+            cus = shmem.get_cu_count()
+            for groups in (cus, cus * 3 // 2, cus * 2, cus * 3):
+                fs = flag_sets[:13]
+                for f in fs:
+                    for r in range(ws):
+                        ops.signal_tiles(shmem.on_rank(f, r), hb, total_tiles, r, ws)
+                for f in fs[:3]:
+                    ops.one_shot_reduce(c, out, f, hb, 0, ws, BLK_M, BLK_N, args.gsize_m, num_sms=groups)
+                torch.cuda.synchronize()
+                s.record()
+                for f in fs[3:]:
+                    ops.one_shot_reduce(c, out, f, hb, 0, ws, BLK_M, BLK_N, args.gsize_m, num_sms=groups)
+                e.record()
+                torch.cuda.synchronize()
+                sweep[str(groups)] = round(rbytes / (s.elapsed_time(e) / 10 * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+            result["reduce"]["frac_by_groups"] = sweep
+
+    if not args.no_context:
+        # (after the two headline measurements: seconds of probes at the power cap in front of the reduce's
+        # thirty launches would be measured with them)
+        result["context"] = context_figures(a, b, c_global, flops, gemm_on)
 
     if args.copy_calibration:
         # ws=1, fp32 -> fp32: the reduce kernel degenerates to a plain tiled copy
