@@ -120,11 +120,20 @@ struct Mfma<IRIS_DTYPE_F16> {
   }
 };
 
-template <int DT_, int CM_, int CN_, int BK_, int WM_, int WN_, int S_, bool DMA_>
+// LW_: waves that only fetch.  With one wave per SIMD a wave that is held up
+// at the issue of a load (the memory pipeline takes a wave's loads at the
+// rate it delivers them) runs no MFMA meanwhile, and the K loop costs the sum
+// of fetch and multiply time.  LW_ = 4 adds one wave per SIMD that does
+// nothing but issue the stage loads and wait for them; the WM x WN waves then
+// issue no memory instruction in the K loop.
+template <int DT_, int CM_, int CN_, int BK_, int WM_, int WN_, int S_, bool DMA_, int LW_ = 0>
 struct GemmCfg {
   static constexpr int DT = DT_, CM = CM_, CN = CN_, BK = BK_, WM = WM_, WN = WN_, S = S_;
   static constexpr bool DMA = DMA_;
-  static constexpr int NW = WM * WN, NT = NW * 64;
+  static constexpr int NW = WM * WN, NT = NW * 64;  // the waves (threads) that multiply and store
+  static constexpr int LW = LW_;
+  static constexpr int NL = LW ? LW : NW;           // the waves that fetch
+  static constexpr int THREADS = (NW + LW) * 64;    // launch size
   static constexpr int TM = CM / WM, TN = CN / WN;
   static constexpr int IM = TM / 16, IN = TN / 16;  // 16x16 MFMA blocks of the wave tile
   static constexpr int CPR = BK / 8;    // 16-byte chunks per slab row
@@ -132,8 +141,8 @@ struct GemmCfg {
   static constexpr int RPB = 64 / CPR;  // slab rows per 1 KiB block (one wave-wide DMA)
   static constexpr int A_BYTES = CM * BK * 2, B_BYTES = CN * BK * 2;
   static constexpr int STAGE = A_BYTES + B_BYTES;
-  static constexpr int A_LOADS = CM * CPR / NT, B_LOADS = CN * CPR / NT;
-  static constexpr int L = A_LOADS + B_LOADS;
+  static constexpr int A_LOADS = CM * CPR / (NL * 64), B_LOADS = CN * CPR / (NL * 64);
+  static constexpr int L = A_LOADS + B_LOADS;  // loads of a fetching wave per stage
   static constexpr int KSUB = BK / 32;  // K-substeps (one MFMA depth) per stage
   // Every LDS-DMA tile with two substeps a stage has a split-K build.  In the
   // tiles with at most 64 accumulator registers a lane the first part of a tile
@@ -152,8 +161,9 @@ struct GemmCfg {
   static constexpr int ERPB = 128 / TN;    // scratch rows per 256 bytes
   static constexpr int LDS_BYTES = S * STAGE + NW * WS_BYTES;
   static_assert(CM % (WM * 32) == 0 && CN % (WN * 32) == 0, "wave tile must be a multiple of 32x32");
-  static_assert(BK == 32 || BK == 64, "BK");
-  static_assert((CM * CPR) % NT == 0 && (CN * CPR) % NT == 0, "slab must split evenly over lanes");
+  static_assert(BK == 32 || BK == 64 || BK == 128, "BK");
+  static_assert((CM * CPR) % (NL * 64) == 0 && (CN * CPR) % (NL * 64) == 0, "slab must split evenly over lanes");
+  static_assert(LW == 0 || (DMA && NW + LW <= 8), "fetching waves: LDS-DMA tiles of at most eight waves in all");
   static_assert(A_LOADS >= 1 && B_LOADS >= 1, "too many waves for this slab");
   static_assert((S & (S - 1)) == 0 && S >= 1, "ring depth must be a power of two");
   static_assert(!DMA || S >= 2, "the DMA ring needs a stage being read and one in flight");
@@ -280,16 +290,16 @@ __device__ inline IRIS_GLOBAL P* rank_ptr(const GemmKArgs& p, P* ptr, int r) {
 // Slab loader
 // ---------------------------------------------------------------------------
 
-// Per-item loader state.  Lane `lane` of wave `wave` fetches, for load `i`,
-// the 16-byte chunk that lands at byte  blk*1024 + lane*16  of the slab,
-// blk = i*NW + wave.  That position is (row, physical chunk); the chunk of the
+// Per-item loader state.  Lane `lane` of fetching wave `wave` (of NL) fetches,
+// for load `i`, the 16-byte chunk that lands at byte  blk*1024 + lane*16  of
+// the slab, blk = i*NL + wave.  That position is (row, physical chunk); the chunk of the
 // row it must hold is  pc ^ ((row / RP) % CPR).
 template <class Cfg>
 struct Loader {
   __amdgpu_buffer_rsrc_t ra, rb;
   // Byte offset, at k0 == 0, of the 16-byte chunk this lane fetches with the
   // first A load and the first B load of a slab; load i of an operand is
-  // i * NW * RPB rows further down (step_a / step_b bytes).  Rows below the
+  // i * NL * RPB rows further down (step_a / step_b bytes).  Rows below the
   // matrix edge lie past the end of the buffer descriptor and read as zero.
   // For the one K-step that can hold chunks past K, the K loop's last, the
   // offsets of those lanes are parked out of range when the load cursor
@@ -301,7 +311,7 @@ struct Loader {
 
   // The chunk of the row that a lane fetches is the same for every load:
   // the swizzle period divides the rows between two loads of a wave.
-  static_assert((Cfg::NW * Cfg::RPB / Cfg::RP) % Cfg::CPR == 0, "the lane's chunk must not depend on the load");
+  static_assert((Cfg::NL * Cfg::RPB / Cfg::RP) % Cfg::CPR == 0, "the lane's chunk must not depend on the load");
   // first k of the chunk that this lane fetches at k0 == 0
   __device__ static inline int chunk_k(int wave, int lane) {
     const int row = wave * Cfg::RPB + lane / Cfg::CPR;
@@ -323,8 +333,8 @@ struct Loader {
     const int row = wave * Cfg::RPB + lane / Cfg::CPR, ck = chunk_k(wave, lane);
     va = (uint32_t)(((int64_t)row * p.sam + ck) * 2);
     vb = (uint32_t)(((int64_t)row * p.sbn + ck) * 2);
-    step_a = (int)((int64_t)Cfg::NW * Cfg::RPB * p.sam * 2);
-    step_b = (int)((int64_t)Cfg::NW * Cfg::RPB * p.sbn * 2);
+    step_a = (int)((int64_t)Cfg::NL * Cfg::RPB * p.sam * 2);
+    step_b = (int)((int64_t)Cfg::NL * Cfg::RPB * p.sbn * 2);
     before_step(k, wave, lane);
   }
   // The load cursor is about to load step `k`: park the chunks past K.
@@ -343,7 +353,7 @@ struct Loader {
     const bool isA = i < Cfg::A_LOADS;
     const int j = isA ? i : i - Cfg::A_LOADS;
     const int k0 = k * Cfg::BK;
-    IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + (j * Cfg::NW + wave) * 1024;
+    IRIS_LDS char* dst = stage + (isA ? 0 : Cfg::A_BYTES) + (j * Cfg::NL + wave) * 1024;
     // (a parked offset stays out of range: j * step is far below 2 GiB)
     const uint32_t off = isA ? va + (uint32_t)(j * step_a) : vb + (uint32_t)(j * step_b);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(isA ? ra : rb, (IRIS_LDS void*)dst, 16, off, k0 * 2, 0, 0);
@@ -975,7 +985,7 @@ __device__ inline void fused_reduce_tile(const GemmKArgs& p, const Item& it, int
 // other ranks, wait for the tile's own flag, reduce it over all ranks and
 // store the result, tile by tile, while other programs are in their K loops.
 template <class Cfg, int OP, int ODT, bool SPLIT = false, bool FUSED = false>
-__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::WPE, Cfg::WPE))) void
+__global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(Cfg::WPE, Cfg::WPE))) void
 gemm_persistent_kernel(const GemmKArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   IRIS_LDS char* lds = (IRIS_LDS char*)lds_raw;
@@ -983,6 +993,13 @@ gemm_persistent_kernel(const GemmKArgs p) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
+  // Roles (wave-uniform).  Every wave runs the same control flow, so every
+  // barrier below is met by all of them; only the work is told apart: the
+  // first NW waves multiply and store, the fetching waves (if the tile has
+  // any; otherwise every wave does both) issue the stage loads.
+  const bool worker = Cfg::LW == 0 || wave < Cfg::NW;
+  const bool fetcher = Cfg::LW == 0 || wave >= Cfg::NW;
+  const int fwave = Cfg::LW == 0 ? wave : wave - Cfg::NW;  // index among the fetching waves
   int pid;
   if (p.xcd_per > 0) {
     // workgroups are dealt to the XCDs round-robin: this one is number j on XCD x
@@ -1070,7 +1087,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
           q.vec_out = 1;
           q.sys = 0;
           q.heap_bases = nullptr;
-          store_acc<Cfg, OP_STORE32, IRIS_DTYPE_F32>(q, acc, ws, wm * Cfg::TM, wn * Cfg::TN, Cfg::CM, Cfg::CN, lane);
+          if (worker)
+            store_acc<Cfg, OP_STORE32, IRIS_DTYPE_F32>(q, acc, ws, wm * Cfg::TM, wn * Cfg::TN, Cfg::CM, Cfg::CN, lane);
         }
         IRIS_WAIT_VMCNT(0);  // this wave's part of the partial has been written
         __syncthreads();
@@ -1080,7 +1098,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
         }
         __syncthreads();
         const int ok = *okslot;
-        if (ok)
+        if (ok && worker)
           slice_epilogue<Cfg, OP, ODT>(p, c_it, slot0, parts, part * Cfg::CM / parts, (part + 1) * Cfg::CM / parts,
                                        tid);
         IRIS_WAIT_VMCNT(0);  // this wave's stores of the slice have completed
@@ -1107,7 +1125,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       if (kr.part != 0) {
         // not the owner: leave the partial, raise the lock once every wave's
         // stores have completed, and move on
-        dump_partial<Cfg>(p, acc, kr.slot, tid);
+        if (worker) dump_partial<Cfg>(p, acc, kr.slot, tid);
         IRIS_WAIT_VMCNT(0);
         __syncthreads();
         if (tid == 0) flag_add_relaxed((IRIS_GLOBAL int32_t*)(p.locks + kr.slot), 1, false);
@@ -1123,12 +1141,15 @@ gemm_persistent_kernel(const GemmKArgs p) {
         ok = wait_tile_flag((IRIS_GLOBAL int32_t*)(p.locks + kr.slot + tid), 2, false, p.timeout, p.status) ? 1 : 0;
       if (__syncthreads_and(ok)) {
         constexpr int GROUP = Cfg::IM * Cfg::IN * 4 <= 16 ? 4 : Cfg::IM * Cfg::IN * 4 <= 32 ? 2 : 1;
-        for (int q = 1; q < parts; q += GROUP) add_partials<Cfg, GROUP>(p, acc, kr.slot, q, parts, tid);
+        if (worker)
+          for (int q = 1; q < parts; q += GROUP) add_partials<Cfg, GROUP>(p, acc, kr.slot, q, parts, tid);
       }
       }
     }
-    const bool fast = store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN,
-                                              c_it.m_end, c_it.n_end, lane);
+    bool fast = true;  // (a fetching wave has no stores to count)
+    if (worker)
+      fast = store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end, c_it.n_end,
+                                     lane);
     if constexpr (FUSED) {
       static_assert(!SPLIT && (OP == OP_STORE16 || OP == OP_STORE32), "the in-program reduce follows a plain store");
       if (c_it.last_sub) {
@@ -1151,7 +1172,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
         if (ok) {
           // rows in flight per lane (the accumulators' registers are free by now)
           constexpr int UN = 4;
-          if (p.sys)
+          if (!worker) {
+          } else if (p.sys)
             fused_reduce_tile<IN_DT, Cfg::NT, UN, true>(p, c_it, tid);
           else
             fused_reduce_tile<IN_DT, Cfg::NT, UN, false>(p, c_it, tid);
@@ -1204,33 +1226,37 @@ gemm_persistent_kernel(const GemmKArgs p) {
           const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, l_item, nk);
           l_k = kr.k_begin;
           l_kend = kr.k_end;
-          ld.setup(p, l_it, wave, lane, l_k);
+          ld.setup(p, l_it, fwave, lane, l_k);
         } else {
           l_k = 0;
           l_kend = nk;
           ld.park();  // nothing left to load
         }
       } else {
-        ld.before_step(l_k, wave, lane);
+        ld.before_step(l_k, fwave, lane);
       }
     };
     Frags<Cfg> fr;
     if (total_steps > 0) {
-      l_it = decode_item<Cfg, SPLIT>(p, sr, pid, 0);
-      const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, 0, nk);
-      l_k = kr.k_begin;
-      l_kend = kr.k_end;
-      ld.setup(p, l_it, wave, lane, l_k);
+      if (fetcher) {
+        l_it = decode_item<Cfg, SPLIT>(p, sr, pid, 0);
+        const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, 0, nk);
+        l_k = kr.k_begin;
+        l_kend = kr.k_end;
+        ld.setup(p, l_it, fwave, lane, l_k);
 #pragma unroll
-      for (int s = 0; s < Cfg::S; ++s) {
-        ld.issue(p, lds + s * Cfg::STAGE, l_k, wave);
-        advance_load_cursor();
+        for (int s = 0; s < Cfg::S; ++s) {
+          ld.issue(p, lds + s * Cfg::STAGE, l_k, fwave);
+          advance_load_cursor();
+        }
+        // stage 0 has landed once at most S-1 younger slabs are outstanding
+        IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 1));
       }
-      // stage 0 has landed once at most S-1 younger slabs are outstanding
-      IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 1));
       block_barrier_raw();
-      load_all<Cfg>(lds + a_row_off + xoff[0], lds + Cfg::A_BYTES + b_row_off + xoff[0], fr, 0);
-      IRIS_WAIT_LGKMCNT0();
+      if (worker) {
+        load_all<Cfg>(lds + a_row_off + xoff[0], lds + Cfg::A_BYTES + b_row_off + xoff[0], fr, 0);
+        IRIS_WAIT_LGKMCNT0();
+      }
     }
 
     // One K-step (global step number g).  FIRST: the tile's first step, whose
@@ -1250,36 +1276,46 @@ gemm_persistent_kernel(const GemmKArgs p) {
       constexpr bool FIRST = decltype(first_tag)::value;
       constexpr int PAR = decltype(par_tag)::value;
       const IRIS_LDS char* stage = lds + (g & (Cfg::S - 1)) * Cfg::STAGE;
+      if (worker) {
 #pragma unroll
-      for (int kk = 0; kk < Cfg::KSUB - 1; ++kk) {
-        const int cb = (PAR + kk) & 1;
-        const IRIS_LDS char* sA = stage + a_row_off + xoff[kk + 1];
-        const IRIS_LDS char* sB = stage + Cfg::A_BYTES + b_row_off + xoff[kk + 1];
+        for (int kk = 0; kk < Cfg::KSUB - 1; ++kk) {
+          const int cb = (PAR + kk) & 1;
+          const IRIS_LDS char* sA = stage + a_row_off + xoff[kk + 1];
+          const IRIS_LDS char* sB = stage + Cfg::A_BYTES + b_row_off + xoff[kk + 1];
 #pragma unroll
-        for (int i = 0; i < Cfg::IM; ++i) {
-          if (FIRST && kk == 0)
-            mma_row<Cfg, true>(acc, fr, cb, i);
-          else
-            mma_row<Cfg, false>(acc, fr, cb, i);
-          fr.a[i] = load_a<Cfg>(sA, i);
-          load_b_share<Cfg>(sB, i, fr.b[cb ^ 1]);
-          __builtin_amdgcn_sched_barrier(0);
+          for (int i = 0; i < Cfg::IM; ++i) {
+            if (FIRST && kk == 0)
+              mma_row<Cfg, true>(acc, fr, cb, i);
+            else
+              mma_row<Cfg, false>(acc, fr, cb, i);
+            fr.a[i] = load_a<Cfg>(sA, i);
+            load_b_share<Cfg>(sB, i, fr.b[cb ^ 1]);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       }
       {
         constexpr int kk = Cfg::KSUB - 1;
         constexpr int cb = (PAR + kk) & 1;
         constexpr bool F = FIRST && kk == 0;
-        mma_row<Cfg, F>(acc, fr, cb, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        // this wave's reads of stage g have returned (they were issued a
-        // substep ago), so the stage may be refilled after the barrier
-        IRIS_WAIT_LGKMCNT0();
+        if (worker) {
+          mma_row<Cfg, F>(acc, fr, cb, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          // this wave's reads of stage g have returned (they were issued a
+          // substep ago), so the stage may be refilled after the barrier
+          IRIS_WAIT_LGKMCNT0();
+        }
         // hand-over of stage g+1: wait for this wave's part of its slab
         // (S-2 younger slabs may stay in flight), then meet the other waves
         const int pend = __builtin_amdgcn_readfirstlane(pending_tile);
         const int skip = __builtin_amdgcn_readfirstlane(pending_skip);
-        if (pend >= 0 && skip == 0) {
+        if constexpr (Cfg::LW != 0) {
+          if (fetcher) {
+            IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
+          } else if (pend >= 0 && skip == 0) {
+            IRIS_WAIT_VMCNT(0);  // the previous tile's stores (all this wave has in flight)
+          }
+        } else if (pend >= 0 && skip == 0) {
           IRIS_WAIT_VMCNT(0);  // the previous tile's stores, too
         } else if (pend >= 0) {
           IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2) + FAST_STORES);  // the stores stay in flight
@@ -1299,22 +1335,34 @@ gemm_persistent_kernel(const GemmKArgs p) {
         const IRIS_LDS char* sA = nstage + a_row_off + xoff[0];
         const IRIS_LDS char* sB = nstage + Cfg::A_BYTES + b_row_off + xoff[0];
         IRIS_LDS char* rstage = lds + (g & (Cfg::S - 1)) * Cfg::STAGE;
-        fr.a[0] = load_a<Cfg>(sA, 0);
-        load_b_share<Cfg>(sB, 0, fr.b[cb ^ 1]);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 1; i < Cfg::IM; ++i) {
-          mma_row<Cfg, F>(acc, fr, cb, i);
-          fr.a[i] = load_a<Cfg>(sA, i);
-          load_b_share<Cfg>(sB, i, fr.b[cb ^ 1]);
-          // every wave is past its reads of stage g: refill it with step g+S,
-          // the L loads shared out over the blocks
-#pragma unroll
-          for (int q = (i - 1) * Cfg::L / (Cfg::IM - 1); q < i * Cfg::L / (Cfg::IM - 1); ++q)
-            ld.issue_at(p, rstage, l_k, wave, q);
+        if (worker) {
+          fr.a[0] = load_a<Cfg>(sA, 0);
+          load_b_share<Cfg>(sB, 0, fr.b[cb ^ 1]);
           __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int i = 1; i < Cfg::IM; ++i) {
+            mma_row<Cfg, F>(acc, fr, cb, i);
+            fr.a[i] = load_a<Cfg>(sA, i);
+            load_b_share<Cfg>(sB, i, fr.b[cb ^ 1]);
+            // every wave is past its reads of stage g: refill it with step g+S,
+            // the L loads shared out over the blocks
+            if constexpr (Cfg::LW == 0) {
+#pragma unroll
+              for (int q = (i - 1) * Cfg::L / (Cfg::IM - 1); q < i * Cfg::L / (Cfg::IM - 1); ++q)
+                ld.issue_at(p, rstage, l_k, wave, q);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
-        advance_load_cursor();
+        if constexpr (Cfg::LW != 0) {
+          // every wave is past its reads of stage g: refill it with step g+S
+          if (fetcher) {
+            ld.issue(p, rstage, l_k, fwave);
+            advance_load_cursor();
+          }
+        } else {
+          advance_load_cursor();
+        }
       }
     };
     // B buffer a step starts with: substeps alternate, so with an odd KSUB

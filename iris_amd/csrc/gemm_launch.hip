@@ -31,6 +31,17 @@ const GemmKernelEntry* entries_for(int dt, int op, int* count) {
   return nullptr;
 }
 
+// The plain build (every wave fetches its share) of the tile shape of `e`, an
+// entry with fetching waves; null if `e` has none or the list holds no such build.
+const GemmKernelEntry* plain_twin(const GemmKernelEntry* list, int count, const GemmKernelEntry& e) {
+  if (e.fetch_waves == 0) return nullptr;
+  for (int i = 0; i < count; ++i)
+    if (list[i].dma && list[i].fetch_waves == 0 && list[i].cm == e.cm && list[i].cn == e.cn && list[i].wm == e.wm &&
+        list[i].wn == e.wn)
+      return &list[i];
+  return nullptr;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // 16-byte vector access on a row-major [rows, cols] view of `es`-byte elements
@@ -107,6 +118,8 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
   if (a.split_handover < IRIS_GEMM_HANDOVER_AUTO || a.split_handover > IRIS_GEMM_HANDOVER_SLICED)
     return hipErrorInvalidValue;
   const int nk = (a.K + pick.bk - 1) / pick.bk;
+  // the rules below were measured on K-steps of 64: `d` such steps to one of this tile
+  const int d = pick.bk > 64 ? pick.bk / 64 : 1;
   if (in_program) {
     // the program that computes a tile also reduces it: K is never shared out
     return (a.split_k > 1 || a.split_k == IRIS_GEMM_SPLIT_STREAM_K) ? hipErrorInvalidValue : hipSuccess;
@@ -120,7 +133,7 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
     // A run of at least four steps keeps the parts of a tile few.
     const int64_t steps = (int64_t)k.total_tiles * nk;
     const int run = (int)(steps / a.num_sms);
-    const bool stream_ok = possible && pick.split_owner && run >= 4 && steps < ((int64_t)1 << 30) &&
+    const bool stream_ok = possible && pick.split_owner && run * d >= 4 && run >= 1 && steps < ((int64_t)1 << 30) &&
                            (nk + run - 1) / run + 1 <= 32;
     if (a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
       if (!stream_ok) return hipErrorInvalidValue;
@@ -133,7 +146,7 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
       // K-steps a program walks through, unsplit
       const int rounds = (k.total_tiles + a.num_sms - 1) / a.num_sms;
       int walk = rounds * nk;
-      if (k.total_tiles * 2 <= a.num_sms && nk >= 16) {
+      if (k.total_tiles * 2 <= a.num_sms && nk * d >= 16) {
         // The hand-over of partials costs about as much as ten K-steps of a
         // small tile: as many parts as there are idle programs, at least four
         // K-steps each, and a K loop shorter than 32 steps is only split in
@@ -141,9 +154,9 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
         // 128 x 128 tiles: 4 parts 16.4 against 19.5 us unsplit at 128 rows,
         // 2 parts 25.9 against 20.2 at 512).
         int sk = a.num_sms / k.total_tiles;
-        if (sk > nk / 4) sk = nk / 4;
+        if (sk > nk * d / 4) sk = nk * d / 4;
         if (sk > 16) sk = 16;
-        if (sk >= 4 || (sk > 1 && nk >= 32)) {
+        if (sk >= 4 || (sk > 1 && nk * d >= 32)) {
           k.split_k = sk;
           walk = (nk + sk - 1) / sk;
         }
@@ -157,8 +170,8 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
       // the unsplit one (132 tiles of 64 steps on 256 programs: -17 %; 176
       // tiles: +9 %; 22-step tiles: +6 to +20 %).
       const bool hidden = run >= nk;
-      if (stream_ok && nk >= 16 && run >= 8 && (int64_t)(run + 1) * 20 <= (int64_t)walk * 17 &&
-          (hidden || (nk >= 32 && (int64_t)(run + 1) * 20 <= (int64_t)rounds * nk * 11))) {
+      if (stream_ok && nk * d >= 16 && run * d >= 8 && (int64_t)(run + 1) * 20 <= (int64_t)walk * 17 &&
+          (hidden || (nk * d >= 32 && (int64_t)(run + 1) * 20 <= (int64_t)rounds * nk * 11))) {
         k.stream_k = 1;
         k.split_k = 1;
       }
@@ -333,6 +346,9 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
     for (int i = 0; i < count && !pick; ++i) {
       const GemmKernelEntry& e = list[i];
       if (!fits(e)) continue;
+      if (plan->in_program && !e.fn_fused) continue;
+      // (a caller's split needs a K-step per part: a tile with a deeper step may not have them)
+      if (a.split_k > 1 && a.split_k > (a.K + e.bk - 1) / e.bk && e.bk > 64) continue;
       if (a.block_m % e.cm != 0 || a.block_n % e.cn != 0) continue;
       // (up to half a tall tile may be padding: its rows cost matrix-core time only, and
       // the tall tiles are the ones whose K range can be shared out over idle programs)
@@ -345,9 +361,9 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
       if ((op == OP_ATOMIC32 || op == OP_ATOMIC16) && e.cm * e.cn > 256 * 128) continue;
       pick = &e;
     }
-    // otherwise the smallest tile that fits, with masked sub-tiles
+    // otherwise the generic tile, with masked sub-tiles
     for (int i = count - 1; i >= 0 && !pick; --i)
-      if (fits(list[i]) && list[i].cm == 64 && list[i].cn == 64) pick = &list[i];
+      if (!list[i].dma && list[i].cm == 64 && list[i].cn == 64) pick = &list[i];
   }
   if (!pick) return hipErrorInvalidValue;
   if (plan->in_program && !pick->fn_fused) return hipErrorInvalidValue;
@@ -383,10 +399,20 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   // flags are.  (64 x 64 tiles, 256 -> 512 programs: [512,1376] x [1376,4096]
   // 25.0 -> 17.8 us, [2048,4096] x [4096,1376] 80 -> 65 us.)
   const int64_t items = (int64_t)k.total_tiles * k.sub_m * k.sub_n;
-  if (!plan->in_program && k.split_k == 1 && pick->lds_bytes * 2 <= 160 * 1024 && a.num_sms >= current_cu_count() &&
-      a.num_sms <= 2 * current_cu_count() && items >= 2 * (int64_t)a.num_sms && !a.mm_begin_timestamp &&
-      !a.mm_end_timestamp)
+  // (Two programs of a tile with fetching waves are slower than one, so such a launch takes
+  // the plain tile of the same shape: [512,1376] x [1376,4096] 20.6 -> 17.1 us.)
+  const GemmKernelEntry* twin = a.variant > 0 ? nullptr : plain_twin(list, count, *pick);
+  const bool two_ok = pick->fetch_waves == 0 || twin;
+  if (!plan->in_program && k.split_k == 1 && two_ok && (twin ? twin : pick)->lds_bytes * 2 <= 160 * 1024 &&
+      a.num_sms >= current_cu_count() && a.num_sms <= 2 * current_cu_count() && items >= 2 * (int64_t)a.num_sms &&
+      !a.mm_begin_timestamp && !a.mm_end_timestamp) {
     k.num_sms = 2 * a.num_sms;
+    if (twin) plan->entry = twin;
+  }
+  // A split launch of a 128-accumulator tile: the fetch state of the `_f4` build spills next
+  // to the hand-over's registers ([128,4096] x [4096,1376] as one 256 x 128 tile row in 16
+  // parts: 24.0 us against the plain tile's 21.2).
+  if (k.split_k != 1 && twin && !pick->split_owner && twin->bk == pick->bk) plan->entry = twin;
   return hipSuccess;
 }
 

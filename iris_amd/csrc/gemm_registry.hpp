@@ -17,7 +17,8 @@ struct GemmKernelEntry {
   bool dma;    // LDS-DMA loader (needs K-contiguous, 16-byte aligned operands)
   bool splitk;  // the kernel can share a tile's K range with other programs
   bool split_owner;  // ... and its first part can add the others' partials itself (needed for stream-K runs)
-  int threads;
+  int threads;        // launch size: the multiplying waves and the fetching waves (if any)
+  int fetch_waves;    // waves that only issue the stage loads (0: every wave fetches its share)
   int lds_bytes;
   GemmKernelFn fn;
   GemmKernelFn fn_split;  // split-K build, or null
@@ -35,7 +36,9 @@ constexpr GemmKernelFn split_fn() {
 
 template <class Cfg, int OP, int ODT>
 constexpr GemmKernelFn fused_fn() {
-  if constexpr (OP == OP_STORE16 || OP == OP_STORE32)
+  // (the tiles with fetching waves have no such build: the reduce wants the registers their
+  // fetch state takes, and the launcher takes the plain tile of the same shape instead)
+  if constexpr ((OP == OP_STORE16 || OP == OP_STORE32) && Cfg::LW == 0)
     return &gemm_persistent_kernel<Cfg, OP, ODT, false, true>;
   else
     return nullptr;
@@ -45,7 +48,7 @@ template <class Cfg, int OP>
 constexpr GemmKernelEntry make_entry(const char* name) {
   constexpr int ODT = (OP == OP_STORE32 || OP == OP_ATOMIC32) ? IRIS_DTYPE_F32 : Cfg::DT;
   return GemmKernelEntry{Cfg::DT, OP,      Cfg::CM, Cfg::CN, Cfg::BK,        Cfg::WM,
-                         Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::SPLIT_OWNER, Cfg::NT, Cfg::LDS_BYTES,
+                         Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::SPLIT_OWNER, Cfg::THREADS, Cfg::LW, Cfg::LDS_BYTES,
                          &gemm_persistent_kernel<Cfg, OP, ODT, false>, split_fn<Cfg, OP, ODT>(), fused_fn<Cfg, OP, ODT>(),
                          name};
 }
@@ -54,46 +57,64 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 // compute tile divides the logical tile (and whose loader fits the operands)
 // wins.  `variant` k > 0 in iris_gemm_args forces entry k-1 (tuning runs).
 // Columns: compute tile CM, CN, BK; waves WM x WN; stages; LDS-DMA loader;
-// whether the tile also has a split-K build (must equal GemmCfg::SPLITK); name.
-#define IRIS_GEMM_VARIANTS(X, DT, OP)                               \
-  X(DT, OP, 256, 256, 64, 2, 4, 2, true, 1, "256x256x64_w2x4_s2")   \
-  X(DT, OP, 256, 128, 64, 2, 2, 2, true, 1, "256x128x64_w2x2_s2")   \
-  X(DT, OP, 128, 256, 64, 1, 4, 2, true, 1, "128x256x64_w1x4_s2")   \
-  X(DT, OP, 128, 128, 64, 2, 2, 4, true, 1, "128x128x64_w2x2_s4")   \
-  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 1, "256x64x64_w4x1_s2")     \
-  X(DT, OP, 64, 64, 64, 2, 2, 4, true, 1, "64x64x64_w2x2_s4")       \
-  X(DT, OP, 64, 64, 32, 2, 2, 1, false, 0, "64x64x32_w2x2_generic")
+// fetching waves; whether the tile also has a split-K build (must equal
+// GemmCfg::SPLITK); name.
+//
+// The four-wave tiles come twice: with one fetching wave per SIMD beside the
+// multiplying one (`_f4`: a K-step then costs the longer of fetch and multiply
+// instead of their sum; [2048,4096] x [4096,1376] in 128 x 128 tiles 48 -> 40 us),
+// and plain, which the launcher takes where the first loses: with the reduce
+// inside the program (no such build), for a split launch of a 128-accumulator
+// tile (its fetch state spills there), and for two programs per CU.
+#define IRIS_GEMM_VARIANTS(X, DT, OP)                                     \
+  X(DT, OP, 256, 256, 64, 2, 4, 2, true, 0, 1, "256x256x64_w2x4_s2")         \
+  X(DT, OP, 256, 128, 64, 2, 2, 2, true, 4, 1, "256x128x64_w2x2_s2_f4")      \
+  X(DT, OP, 128, 256, 64, 1, 4, 2, true, 4, 1, "128x256x64_w1x4_s2_f4")      \
+  X(DT, OP, 128, 128, 64, 2, 2, 4, true, 4, 1, "128x128x64_w2x2_s4_f4")      \
+  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")        \
+  X(DT, OP, 64, 64, 128, 2, 2, 4, true, 4, 1, "64x64x128_w2x2_s4_f4")        \
+  X(DT, OP, 256, 128, 64, 2, 2, 2, true, 0, 1, "256x128x64_w2x2_s2")         \
+  X(DT, OP, 128, 256, 64, 1, 4, 2, true, 0, 1, "128x256x64_w1x4_s2")         \
+  X(DT, OP, 128, 128, 64, 2, 2, 4, true, 0, 1, "128x128x64_w2x2_s4")         \
+  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 0, 1, "256x64x64_w4x1_s2")           \
+  X(DT, OP, 64, 64, 64, 2, 2, 4, true, 0, 1, "64x64x64_w2x2_s4")             \
+  X(DT, OP, 64, 64, 32, 2, 2, 1, false, 0, 0, "64x64x32_w2x2_generic")
 
 // extra variants, compiled for the bf16 store op only (tuning runs, and the
 // one-substep stage whose fragment buffers alternate from step to step)
-#define IRIS_GEMM_TUNING_VARIANTS(X, DT, OP)                        \
-  X(DT, OP, 256, 128, 32, 2, 4, 4, true, 0, "256x128x32_w2x4_s4")   \
-  X(DT, OP, 256, 128, 64, 2, 4, 2, true, 1, "256x128x64_w2x4_s2")   \
-  X(DT, OP, 128, 256, 64, 2, 4, 2, true, 1, "128x256x64_w2x4_s2")   \
-  X(DT, OP, 128, 128, 32, 2, 2, 4, true, 0, "128x128x32_w2x2_s4")
+#define IRIS_GEMM_TUNING_VARIANTS(X, DT, OP)                              \
+  X(DT, OP, 256, 128, 32, 2, 4, 4, true, 0, 0, "256x128x32_w2x4_s4")         \
+  X(DT, OP, 256, 128, 64, 2, 4, 2, true, 0, 1, "256x128x64_w2x4_s2")         \
+  X(DT, OP, 128, 256, 64, 2, 4, 2, true, 0, 1, "128x256x64_w2x4_s2")         \
+  X(DT, OP, 128, 128, 32, 2, 2, 4, true, 0, 0, "128x128x32_w2x2_s4")         \
+  X(DT, OP, 64, 64, 64, 2, 2, 4, true, 4, 1, "64x64x64_w2x2_s4_f4")
 
-#define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, SPLIT, NAME) \
-  make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP>(NAME),
+#define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, SPLIT, NAME) \
+  make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP>(NAME),
 
 // Explicit instantiation of an entry's kernels.  Taking their addresses in
 // make_entry should be enough, but with the plain and the split-K build of a
 // tile in one translation unit the compiler's host pass has been seen to
 // reference one of the two without emitting it.
 #define IRIS_GEMM_ODT(DT, OP) (((OP) == OP_STORE32 || (OP) == OP_ATOMIC32) ? IRIS_DTYPE_F32 : (DT))
-#define IRIS_GEMM_INSTANTIATE_SPLIT_0(DT, OP, CM, CN, BK, WM, WN, S, DMA) \
-  static_assert(!GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>::SPLITK, "split-K column of the variant table");
-#define IRIS_GEMM_INSTANTIATE_SPLIT_1(DT, OP, CM, CN, BK, WM, WN, S, DMA)                                  \
-  static_assert(GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>::SPLITK, "split-K column of the variant table"); \
-  template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP,           \
+#define IRIS_GEMM_INSTANTIATE_SPLIT_0(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW) \
+  static_assert(!GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>::SPLITK, "split-K column of the variant table");
+#define IRIS_GEMM_INSTANTIATE_SPLIT_1(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW)                                  \
+  static_assert(GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>::SPLITK, "split-K column of the variant table"); \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP,           \
                                                   IRIS_GEMM_ODT(DT, OP), true>(const GemmKArgs);
-#define IRIS_GEMM_INSTANTIATE(DT, OP, CM, CN, BK, WM, WN, S, DMA, SPLIT, NAME)                    \
-  template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP,    \
+#define IRIS_GEMM_INSTANTIATE(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, SPLIT, NAME)                    \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP,    \
                                                   IRIS_GEMM_ODT(DT, OP), false>(const GemmKArgs); \
-  IRIS_GEMM_INSTANTIATE_SPLIT_##SPLIT(DT, OP, CM, CN, BK, WM, WN, S, DMA)
+  IRIS_GEMM_INSTANTIATE_SPLIT_##SPLIT(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW)
 // the store epilogues' build with the one-shot reduce inside the program
-#define IRIS_GEMM_INSTANTIATE_FUSED(DT, OP, CM, CN, BK, WM, WN, S, DMA, SPLIT, NAME)           \
+#define IRIS_GEMM_INSTANTIATE_FUSED(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, SPLIT, NAME) \
+  IRIS_GEMM_INSTANTIATE_FUSED_##LW(DT, OP, CM, CN, BK, WM, WN, S, DMA)
+#define IRIS_GEMM_INSTANTIATE_FUSED_0(DT, OP, CM, CN, BK, WM, WN, S, DMA)                     \
   template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP, \
                                                   IRIS_GEMM_ODT(DT, OP), false, true>(const GemmKArgs);
+#define IRIS_GEMM_INSTANTIATE_FUSED_2(DT, OP, CM, CN, BK, WM, WN, S, DMA)
+#define IRIS_GEMM_INSTANTIATE_FUSED_4(DT, OP, CM, CN, BK, WM, WN, S, DMA)
 
 #define IRIS_GEMM_DECLARE(TAG) const GemmKernelEntry* gemm_entries_##TAG(int* count);
 IRIS_GEMM_DECLARE(bf16_store16)
