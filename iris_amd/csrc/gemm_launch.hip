@@ -170,7 +170,10 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
       // the unsplit one (132 tiles of 64 steps on 256 programs: -17 %; 176
       // tiles: +9 %; 22-step tiles: +6 to +20 %).
       const bool hidden = run >= nk;
-      if (stream_ok && nk * d >= 16 && run * d >= 8 && (int64_t)(run + 1) * 20 <= (int64_t)walk * 17 &&
+      // (With more tiles than programs it lost wherever it was measured: 352 tiles of
+      // 128 x 64 on 256 programs 80 us against 54 unsplit.)
+      if (stream_ok && k.total_tiles <= a.num_sms && nk * d >= 16 && run * d >= 8 &&
+          (int64_t)(run + 1) * 20 <= (int64_t)walk * 17 &&
           (hidden || (nk * d >= 32 && (int64_t)(run + 1) * 20 <= (int64_t)rounds * nk * 11))) {
         k.stream_k = 1;
         k.split_k = 1;

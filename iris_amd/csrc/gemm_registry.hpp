@@ -72,6 +72,8 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   X(DT, OP, 128, 256, 64, 1, 4, 2, true, 4, 1, "128x256x64_w1x4_s2_f4")      \
   X(DT, OP, 128, 128, 64, 2, 2, 4, true, 4, 1, "128x128x64_w2x2_s4_f4")      \
   X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")        \
+  X(DT, OP, 128, 64, 64, 2, 2, 4, true, 4, 1, "128x64x64_w2x2_s4_f4")        \
+  X(DT, OP, 64, 128, 64, 2, 2, 4, true, 4, 1, "64x128x64_w2x2_s4_f4")        \
   X(DT, OP, 64, 64, 128, 2, 2, 4, true, 4, 1, "64x64x128_w2x2_s4_f4")        \
   X(DT, OP, 256, 128, 64, 2, 2, 2, true, 0, 1, "256x128x64_w2x2_s2")         \
   X(DT, OP, 128, 256, 64, 1, 4, 2, true, 0, 1, "128x256x64_w1x4_s2")         \

@@ -231,8 +231,13 @@ def test_choice_of_kernel(shmem):
     assert plan(a, b, cg, 16, 16) == FEW
     # the persistent kernels on request
     assert plan(a, b, cg, 64, 64, locks=locks, variant=ops.VARIANT_PERSISTENT) == "64x64x128_w2x2_s4_f4"
-    assert plan(a, b, cg, 64, 64, locks=locks, variant=6) == "64x64x128_w2x2_s4_f4"
-    assert plan(a, b, cg, 64, 64, locks=locks, variant=11) == "64x64x64_w2x2_s4"
+    names = {}
+    v = 1
+    while (name := ops.gemm_variant_name(dtype, False, False, v)) is not None:
+        names[name] = v
+        v += 1
+    for name in ("64x64x128_w2x2_s4_f4", "64x64x64_w2x2_s4"):
+        assert plan(a, b, cg, 64, 64, locks=locks, variant=names[name]) == name
     # a logical tile that does not cover the rows, or is no multiple of 16 columns
     assert plan(a, b, cg, 8, 64, locks=locks) != FEW
     assert plan(a, b, cg, 64, 40, locks=locks) != FEW
