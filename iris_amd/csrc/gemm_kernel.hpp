@@ -662,16 +662,22 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
 // Publish a finished logical tile: +1 on the tile's flag of every rank
 // (flag_mode 1, the ready flag of the scatter epilogue) or of every *other*
 // rank (flag_mode 2, the ONE_SHOT producer signal,
-// gemm_one_shot_all_reduce.py:207-218, sem="release").  One thread calls it
-// after every wave of the group has waited for its stores of the tile to
-// complete and the group has passed a barrier.  Those stores were
+// gemm_one_shot_all_reduce.py:207-218, sem="release").  One wave calls it, all
+// 64 lanes, after every wave of the group has waited for its stores of the
+// tile to complete and the group has passed a barrier.  Those stores were
 // write-through at the flag's scope, so they are already visible there and
 // the increment itself can be relaxed: it is ordered after them by the waits.
-__device__ inline void publish_tile(const GemmKArgs& p, int tile_id) {
-#pragma nounroll
-  for (int r = 0; r < p.ws; ++r) {
+// Lane l takes ranks l, l + 64, ...: the ranks' heap bases come in with one
+// vector load and the increments leave together (one thread walking the ranks
+// waits for a scalar load per rank: 0.8 us for eight).
+__device__ inline void publish_tile(const GemmKArgs& p, int tile_id, int lane) {
+  IRIS_GLOBAL int32_t* own = (IRIS_GLOBAL int32_t*)(p.flags + tile_id);
+  for (int r = lane; r < p.ws; r += 64) {
     if (p.flag_mode == 2 && r == p.cur_rank) continue;
-    flag_add_relaxed(rank_ptr(p, p.flags + tile_id, r), 1, p.sys != 0);
+    IRIS_GLOBAL int32_t* f = own;
+    if (r != p.cur_rank && p.heap_bases != nullptr)
+      f = translate(p.flags + tile_id, p.heap_bases[p.cur_rank], p.heap_bases[r]);
+    flag_add_relaxed(f, 1, p.sys != 0);
   }
 }
 
@@ -1066,7 +1072,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       // a one-step tile: the previous tile has not been published yet
       IRIS_WAIT_VMCNT(0);
       __syncthreads();
-      if (tid == 0) publish_tile(p, pending_tile);
+      if (wave == 0) publish_tile(p, pending_tile, lane);
       pending_tile = -1;
     }
     if constexpr (SPLIT) {
@@ -1103,14 +1109,18 @@ gemm_persistent_kernel(const GemmKArgs p) {
                                        tid);
         IRIS_WAIT_VMCNT(0);  // this wave's stores of the slice have completed
         __syncthreads();     // (and okslot is scratch again)
-        if (tid == 0 && ok) {
+        if (wave == 0 && ok) {
           IRIS_GLOBAL int32_t* done = (IRIS_GLOBAL int32_t*)(p.locks + slot0 + 1);
-          const int before = __hip_atomic_fetch_add(done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          int before = 0;
+          if (lane == 0) before = __hip_atomic_fetch_add(done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          before = __builtin_amdgcn_readfirstlane(before);
           if (before == parts - 1) {
             // every slice is in memory: publish, and leave both counters at 0
-            if (p.flag_mode != 0) publish_tile(p, c_it.tile_id);
-            flag_add_relaxed(done, -parts, false);
-            flag_add_relaxed((IRIS_GLOBAL int32_t*)(p.locks + slot0), -parts, false);
+            if (p.flag_mode != 0) publish_tile(p, c_it.tile_id, lane);
+            if (lane == 0) {
+              flag_add_relaxed(done, -parts, false);
+              flag_add_relaxed((IRIS_GLOBAL int32_t*)(p.locks + slot0), -parts, false);
+            }
           }
         }
         if (p.ts_end && tid == 0)
@@ -1159,8 +1169,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
         __syncthreads();
         int ok = 1;
         if (p.ws > 1) {
+          if (wave == 0) publish_tile(p, c_it.tile_id, lane);  // +1 on every other rank (:207-218)
           if (tid == 0) {
-            publish_tile(p, c_it.tile_id);  // +1 on every other rank (:207-218)
             *slot = wait_tile_flag((IRIS_GLOBAL int32_t*)(p.flags + c_it.tile_id), p.ws, p.sys != 0, p.timeout,
                                    p.status)
                         ? 1
@@ -1191,7 +1201,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       } else if (p.flag_mode != 0) {
         IRIS_WAIT_VMCNT(0);  // this wave's stores of the tile have completed
         __syncthreads();
-        if (tid == 0) publish_tile(p, c_it.tile_id);
+        if (wave == 0) publish_tile(p, c_it.tile_id, lane);
       }
       if (p.ts_end && tid == 0)
         __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + c_it.tile_id),
@@ -1325,7 +1335,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
         block_barrier_raw();
         if (pend >= 0) {
           if (skip == 0) {
-            if (tid == 0) publish_tile(p, pend);
+            if (wave == 0) publish_tile(p, pend, lane);
             pending_tile = -1;
           } else {
             pending_skip = 0;
@@ -1417,7 +1427,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
   if (pending_tile >= 0) {
     IRIS_WAIT_VMCNT(0);
     __syncthreads();
-    if (tid == 0) publish_tile(p, pending_tile);
+    if (wave == 0) publish_tile(p, pending_tile, lane);
   }
 }
 

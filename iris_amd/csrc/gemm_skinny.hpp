@@ -177,18 +177,21 @@ gemm_skinny_kernel(const GemmKArgs p) {
   // seen its own complete, the group's part of the tile is visible there.
   IRIS_WAIT_VMCNT(0);
   __syncthreads();
-  if (tid == 0) {
+  if (wave == 0) {
     const int pid_n = n0 / p.BN;
     const int tile_id = tile_id_of(0, pid_n, p.num_pid_m, p.num_pid_n, p.G);
     const int cols = min(p.N, (pid_n + 1) * p.BN) - pid_n * p.BN;
     const int parts = ((cols + SKINNY_COLS - 1) / SKINNY_COLS) * gridDim.y;
-    bool last = true;
+    int last = 1;
     if (parts > 1) {
       IRIS_GLOBAL int32_t* cnt = (IRIS_GLOBAL int32_t*)(p.locks + tile_id);
-      last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == parts - 1;
-      if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+      if (lane == 0) {
+        last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == parts - 1;
+        if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+      }
+      last = __builtin_amdgcn_readfirstlane(last);
     }
-    if (last) publish_tile(p, tile_id);
+    if (last) publish_tile(p, tile_id, lane);
   }
 }
 
