@@ -329,6 +329,23 @@ def run_decoder(args, emit=True):
     hb = shmem.get_heap_bases()
     g = torch.Generator().manual_seed(123)
     rows = []
+    # the kernel builds by name: a four-wave tile comes with fetching waves ("_f4") and plain
+    variants, v = {}, 1
+    while (vname := ops.gemm_variant_name(torch.bfloat16, False, False, v)) is not None:
+        variants.setdefault(vname, v)
+        v += 1
+
+    def plain_build_of(kernel):
+        """Variant number of the build of `kernel`'s tile shape and wave layout in which every wave fetches its
+        share of the operands, or None if `kernel` is such a build already."""
+        base = kernel.split("+")[0]
+        if not base.endswith("_f4"):
+            return None
+        shape, waves = base.split("x")[:2], base.split("_")[1]
+        for cand, num in variants.items():
+            if not cand.endswith("_f4") and cand.split("x")[:2] == shape and cand.split("_")[1] == waves:
+                return num
+        return None
     for Mt in [int(t) for t in args.decoder_m.split(",")]:
         off = shmem.heap_offset
         x = shmem.zeros((Mt, hidden), dtype=torch.bfloat16)
@@ -355,7 +372,7 @@ def run_decoder(args, emit=True):
             shapes = [tuple(int(v) for v in args.decoder_tiles.lower().split("x"))]
         elif ref_tile not in shapes:
             shapes.append(ref_tile)
-        best, at_ref = {}, {}
+        best, at_ref, plain_at = {}, {}, {}
         for bm, bn in shapes:
             t_up = ops.cdiv(Mt, bm) * ops.cdiv(ffn, bn)
             t_dn = ops.cdiv(Mt, bm) * ops.cdiv(hidden, bn)
@@ -372,6 +389,11 @@ def run_decoder(args, emit=True):
                 ops.gemm_launch(x, wg.T, None, shmem.on_rank(gate_all, rank), shmem.on_rank(flags_up, rank), hb, rank,
                                 ws, grid_up, bm, bn, 64, 4, ops.EPI_ALL_SCATTER, notify=True, partials=P, locks=locks,
                                 num_xcds=xcds)
+
+            def up_plain_build():  # gate/up through the build without fetching waves
+                ops.gemm_launch(x, wg.T, None, shmem.on_rank(gate_all, rank), shmem.on_rank(flags_up, rank), hb, rank,
+                                ws, grid_up, bm, bn, 64, 4, ops.EPI_ALL_SCATTER, notify=True, partials=P, locks=locks,
+                                num_xcds=xcds, variant=plain_variant)
 
             def up_one():  # the same GEMM with the launching rank as its only destination (a plain GEMM + flags)
                 ops.gemm_launch(x, wg.T, None, shmem.on_rank(gate_all, rank), shmem.on_rank(flags_up, rank), hb[rank:],
@@ -409,10 +431,17 @@ def run_decoder(args, emit=True):
                                                shmem.on_rank(flags_dn, rank), hb, rank, ws, grid_dn, bm, bn, 64, 6,
                                                ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks),
                     "reduce": "reduce"}
-            for name, fn in (("gate_up", up), ("down", down), ("reduce", reduce), ("gate_up_one", up_one)):
-                if name == "gate_up_one":
+            plain_variant = plain_build_of(kern["gate_up"])
+            runs = [("gate_up", up), ("down", down), ("reduce", reduce), ("gate_up_one", up_one)]
+            if plain_variant is not None:
+                runs.append(("gate_up_plain", up_plain_build))
+            for name, fn in runs:
+                if name in ("gate_up_one", "gate_up_plain"):
                     kern[name], sk[name] = kern["gate_up"], sk["gate_up"]
                 ms = graph_ms(fn, 10, 10)
+                if name == "gate_up_plain":  # kept for the tile that wins the sweep, not a candidate itself
+                    plain_at[(bm, bn)] = ms
+                    continue
                 if (bm, bn) == ref_tile:
                     at_ref[name] = (ms, kern[name], sk[name])
                     if not args.decoder_tiles and bm > max(64, 2 * Mt):
@@ -439,6 +468,10 @@ def run_decoder(args, emit=True):
             # gate/up with one destination instead of eight: what the library's figure below compares with like for
             # like (the scatter writes 8 x the output: 45 MB at 2048 rows, ~7 us at the rate HBM takes stores)
             "gate_up_one_destination_us": round(best["gate_up_one"][0] * 1e3, 2),
+            # gate/up at the winning tile through the build in which every wave fetches its own share of the
+            # operands (no fetching waves); null where the winning kernel is such a build
+            "gate_up_without_fetching_waves_us": (round(plain_at[tuple(best["gate_up"][1])] * 1e3, 2)
+                                                  if tuple(best["gate_up"][1]) in plain_at else None),
             # the vendor library's plain GEMM on the same operands (one destination, no flags), same timing
             "library_gate_up_us": round(graph_ms(lambda: torch.matmul(x, wg.T, out=lib_up), 10, 10) * 1e3, 2),
             "library_down_us": round(graph_ms(lambda: torch.matmul(h, wd.T, out=lib_dn), 10, 10) * 1e3, 2),
@@ -664,6 +697,7 @@ def main():
         dec = run_decoder(args, emit=False)
         keep = ("M", "kernel_up", "split_k_up", "gate_up_us", "gate_up_tflops", "gate_up_weight_GBps", "kernel_down",
                 "split_k_down", "down_us", "down_tflops", "reduce_us", "reduce_GBps", "gate_up_one_destination_us",
+                "gate_up_without_fetching_waves_us",
                 "library_gate_up_us", "library_down_us", "at_reference_default_tile_256x64")
         result["other_workloads"] = {
             "atomic_accumulate": {k: at[k] for k in ("value", "unit", "ms_per_step", "atomic_updates_per_s",
