@@ -60,6 +60,9 @@ def parse():
     ap.add_argument("--zero-operands", action="store_true",
                     help="all-zero A and B: nothing toggles in the matrix cores, the clocks stay up, and the time that "
                          "is left is the kernel's structure (not the metric's workload; the JSON line says so)")
+    ap.add_argument("--decoder-split-k", type=int, default=0,
+                    help="decoder workload: split_k of the two GEMMs (0: the launcher's choice, N > 1: N parts, "
+                         "-1: stream-K)")
     ap.add_argument("--decoder-tiles", default="",
                     help="decoder workload: only this tile shape, as BLK_MxBLK_N (default: a sweep, and the "
                          "reference examples' default tile 256x64 beside it)")
@@ -388,22 +391,23 @@ def run_decoder(args, emit=True):
             def up():
                 ops.gemm_launch(x, wg.T, None, shmem.on_rank(gate_all, rank), shmem.on_rank(flags_up, rank), hb, rank,
                                 ws, grid_up, bm, bn, 64, 4, ops.EPI_ALL_SCATTER, notify=True, partials=P, locks=locks,
-                                num_xcds=xcds)
+                                num_xcds=xcds, split_k=args.decoder_split_k)
 
             def up_plain_build():  # gate/up through the build without fetching waves
                 ops.gemm_launch(x, wg.T, None, shmem.on_rank(gate_all, rank), shmem.on_rank(flags_up, rank), hb, rank,
                                 ws, grid_up, bm, bn, 64, 4, ops.EPI_ALL_SCATTER, notify=True, partials=P, locks=locks,
-                                num_xcds=xcds, variant=plain_variant)
+                                num_xcds=xcds, variant=plain_variant, split_k=args.decoder_split_k)
 
             def up_one():  # the same GEMM with the launching rank as its only destination (a plain GEMM + flags)
                 ops.gemm_launch(x, wg.T, None, shmem.on_rank(gate_all, rank), shmem.on_rank(flags_up, rank), hb[rank:],
                                 0, 1, grid_up, bm, bn, 64, 4, ops.EPI_ALL_SCATTER, notify=True, partials=P, locks=locks,
-                                num_xcds=xcds)
+                                num_xcds=xcds, split_k=args.decoder_split_k)
 
             def down():
                 ops.gemm_launch(h, wd.T, shmem.on_rank(part, rank), shmem.on_rank(out, rank),
                                 shmem.on_rank(flags_dn, rank), hb, rank, ws, grid_dn, bm, bn, 64, 6,
-                                ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks, num_xcds=xcds)
+                                ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks, num_xcds=xcds,
+                                split_k=args.decoder_split_k)
 
             def reduce():
                 ops.one_shot_reduce(shmem.on_rank(part, rank), shmem.on_rank(out, rank),
@@ -419,17 +423,19 @@ def run_decoder(args, emit=True):
             assert torch.allclose(shmem.on_rank(part, rank), ref_dn, rtol=1e-2, atol=1e-2), "down partial differs"
             sk = {"gate_up": ops.gemm_split_k(x, wg.T, None, shmem.on_rank(gate_all, rank),
                                               shmem.on_rank(flags_up, rank), hb, rank, ws, grid_up, bm, bn, 64, 4,
-                                              ops.EPI_ALL_SCATTER, partials=P, locks=locks),
+                                              ops.EPI_ALL_SCATTER, partials=P, locks=locks, split_k=args.decoder_split_k),
                   "down": ops.gemm_split_k(h, wd.T, shmem.on_rank(part, rank), shmem.on_rank(out, rank),
                                            shmem.on_rank(flags_dn, rank), hb, rank, ws, grid_dn, bm, bn, 64, 6,
-                                           ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks),
+                                           ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks,
+                                           split_k=args.decoder_split_k),
                   "reduce": 1}
             kern = {"gate_up": ops.gemm_plan_name(x, wg.T, None, shmem.on_rank(gate_all, rank),
                                                   shmem.on_rank(flags_up, rank), hb, rank, ws, grid_up, bm, bn, 64, 4,
-                                                  ops.EPI_ALL_SCATTER, partials=P, locks=locks),
+                                                  ops.EPI_ALL_SCATTER, partials=P, locks=locks, split_k=args.decoder_split_k),
                     "down": ops.gemm_plan_name(h, wd.T, shmem.on_rank(part, rank), shmem.on_rank(out, rank),
                                                shmem.on_rank(flags_dn, rank), hb, rank, ws, grid_dn, bm, bn, 64, 6,
-                                               ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks),
+                                               ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE, partials=P, locks=locks,
+                                           split_k=args.decoder_split_k),
                     "reduce": "reduce"}
             plain_variant = plain_build_of(kern["gate_up"])
             runs = [("gate_up", up), ("down", down), ("reduce", reduce), ("gate_up_one", up_one)]

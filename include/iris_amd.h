@@ -116,8 +116,9 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
  * in a tile, the stream-K schedule the reference's wrappers describe and size
  * their `P` / `locks` buffers for (matmul_wrapper.py:73-92,
  * images/stream_k.excalidraw.svg) but do not implement.  Needs partials and
- * locks; hipErrorInvalidValue when the launch cannot be cut this way.
- * iris_gemm_split_k reports this value when the launcher chose it itself. */
+ * locks; hipErrorInvalidValue when the launch cannot be cut this way.  Only
+ * taken on request (split_k = 0 chooses between an unsplit and a split-K
+ * launch); iris_gemm_split_k reports this value for such a launch. */
 #define IRIS_GEMM_SPLIT_STREAM_K (-1)
 /* iris_gemm_args.split_handover */
 #define IRIS_GEMM_HANDOVER_AUTO 0

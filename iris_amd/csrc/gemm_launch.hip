@@ -143,9 +143,6 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
         return hipErrorInvalidValue;
       k.split_k = a.split_k;
     } else if (possible) {
-      // K-steps a program walks through, unsplit
-      const int rounds = (k.total_tiles + a.num_sms - 1) / a.num_sms;
-      int walk = rounds * nk;
       if (k.total_tiles * 2 <= a.num_sms && nk * d >= 16) {
         // The hand-over of partials costs about as much as ten K-steps of a
         // small tile: as many parts as there are idle programs, at least four
@@ -158,26 +155,15 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
         if (sk > 16) sk = 16;
         if (sk >= 4 || (sk > 1 && nk * d >= 32)) {
           k.split_k = sk;
-          walk = (nk + sk - 1) / sk;
         }
       }
-      // Stream-K when it shortens that walk by 15 % or more.  With runs of at
-      // least a tile's length a tile spans two runs and the second hands its
-      // part over first thing, long before the owner asks: nothing is lost.
-      // With shorter runs the owner waits for programs that finish when it
-      // does, and more CUs pull operands at once; measured on the decoder
-      // shapes that pays when the walk is long and at least 45 % shorter than
-      // the unsplit one (132 tiles of 64 steps on 256 programs: -17 %; 176
-      // tiles: +9 %; 22-step tiles: +6 to +20 %).
-      const bool hidden = run >= nk;
-      // (With more tiles than programs it lost wherever it was measured: 352 tiles of
-      // 128 x 64 on 256 programs 80 us against 54 unsplit.)
-      if (stream_ok && k.total_tiles <= a.num_sms && nk * d >= 16 && run * d >= 8 &&
-          (int64_t)(run + 1) * 20 <= (int64_t)walk * 17 &&
-          (hidden || (nk * d >= 32 && (int64_t)(run + 1) * 20 <= (int64_t)rounds * nk * 11))) {
-        k.stream_k = 1;
-        k.split_k = 1;
-      }
+      // Stream-K is only taken on request.  With the plain four-wave tiles it beat both the
+      // unsplit and the split launch where the tiles left programs idle and the walk was long
+      // (132 tiles of 64 steps on 256 programs: -17 %).  The tiles with fetching waves made
+      // the K-steps a quarter shorter and left the hand-over as it was: on the same shapes
+      // stream-K now ties with split-K (66 tiles: 27.9 against 27.6 us in three parts) or
+      // loses (88 tiles: 33.2 against 31.9 in two parts; 132 tiles: 41.0 against 37.6 unsplit;
+      // more tiles than programs: 80 against 54).
     }
   } else if (a.split_k > 1 || a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
     return hipErrorInvalidValue;  // forced, but no workspace

@@ -238,10 +238,10 @@ def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size,
 
     ``partials`` / ``locks`` are the wrappers' ``P`` and ``locks`` buffers
     (matmul_wrapper.py:29-31): with them, a launch with far fewer tiles than
-    programs splits each tile's K range over several programs, and a launch
-    whose last round of tiles would leave many programs idle is cut into equal
-    runs of K-steps (stream-K, ``split_k=SPLIT_STREAM_K`` to insist) (``split_k`` 0:
-    the launcher decides, 1: never, n: exactly n).  ``split_handover``: how the
+    programs splits each tile's K range over several programs (``split_k`` 0:
+    the launcher decides, 1: never, n: exactly n); ``split_k=SPLIT_STREAM_K``
+    cuts the launch's K-steps into equal runs that cross tile boundaries
+    (stream-K, on request only).  ``split_handover``: how the
     parts of a split tile meet: ``HANDOVER_OWNER`` (the first part adds the
     others' partials and stores the tile), ``HANDOVER_SLICED`` (every part sums
     and stores its share of the rows) or ``HANDOVER_AUTO``; bit-identical results.

@@ -591,7 +591,7 @@ def test_stream_k_all_scatter(shmem, M, N, K, BM, BN, grid, dtype):
         assert int(locks.abs().max().item()) == 0
 
 
-def test_stream_k_is_chosen_when_the_tiles_leave_programs_idle(shmem):
+def test_stream_k_is_only_taken_on_request(shmem):
     dtype = torch.bfloat16
     A, B = make_ab(1024, 1376, 2048, dtype)
     a, b = to_heap(shmem, A), to_heap(shmem, B)
@@ -603,8 +603,9 @@ def test_stream_k_is_chosen_when_the_tiles_leave_programs_idle(shmem):
         return ops.gemm_split_k(a, b, None, cg, flags, None, 0, 1, grid, BM, BN, 64, 4, ops.EPI_ALL_SCATTER,
                                 partials=partials, locks=locks, **kw)
 
-    assert choice(256, 128, 128) == ops.SPLIT_STREAM_K       # 88 tiles on 256 programs
-    assert choice(64, 128, 128) == 1                         # more tiles than programs: measured slower, not taken
+    assert choice(256, 128, 128) == 2                        # 88 tiles on 256 programs: two parts each
+    assert choice(256, 128, 128, split_k=ops.SPLIT_STREAM_K) == ops.SPLIT_STREAM_K
+    assert choice(64, 128, 128) == 1                         # more tiles than programs
     assert choice(88, 128, 128) == 1                         # one tile each
     assert choice(44, 128, 128) == 1                         # two rounds, both full
     assert choice(256, 128, 128, split_k=1) == 1
