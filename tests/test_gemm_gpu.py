@@ -456,6 +456,72 @@ def test_store_probe_writes_every_groups_region(shmem):
         ops.store_probe(operands, sink, out, tiles, 3, groups)
 
 
+def _fetching_wave_cases():
+    """(epilogue, name with fetching waves, variant, name of the plain build of the same tile and wave layout,
+    variant), from the kernel list each epilogue launches from."""
+    cases = []
+    for epilogue, out_is_f32, atomic in (("scatter16", False, False), ("split_k", False, False),
+                                         ("store32", True, False), ("atomic32", True, True)):
+        names, v = [], 1
+        while (name := ops.gemm_variant_name(torch.bfloat16, out_is_f32, atomic, v)) is not None:
+            names.append(name)
+            v += 1
+        for i, n in enumerate(names):
+            if not n.endswith("_f4"):
+                continue
+            shape, waves = n.split("x")[:2], n.split("_")[1]
+            for j, m in enumerate(names):
+                if not m.endswith("_f4") and "generic" not in m and m.split("x")[:2] == shape and m.split("_")[1] == waves:
+                    cases.append((epilogue, n, i + 1, m, j + 1))
+                    break
+    assert len(cases) >= 20
+    return cases
+
+
+@pytest.mark.parametrize("epilogue,f4_name,f4_variant,plain_name,plain_variant", _fetching_wave_cases())
+def test_build_with_fetching_waves_is_bit_identical_to_the_plain_build(shmem, epilogue, f4_name, f4_variant, plain_name,
+                                                                       plain_variant):
+    """The multiplying waves of a `_f4` build run the plain build's MFMA sequence
+    on the same fragments: whoever issues the loads, and however deep a stage
+    is, the accumulators see the same products in the same order.  Ragged
+    edges, a K that ends inside a K-step, several tiles per program."""
+    dtype = torch.bfloat16
+    M, N, K = 520, 392, 1528  # (twelve 128-deep or twenty-four 64-deep steps: three parts cut K at the same places)
+    A, B = make_ab(M, N, K, dtype, lda=1536, ldb=1544)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    bm, bn = (int(v) for v in f4_name.split("x")[:2])
+    total = ops.cdiv(M, bm) * ops.cdiv(N, bn)
+    got = {}
+    for variant in (f4_variant, plain_variant):
+        flags = shmem.zeros((total,), dtype=torch.int32)
+        if epilogue == "scatter16":
+            out = shmem.zeros((M, N), dtype=dtype)
+            ops.gemm_launch(a, b, None, out, flags, None, 0, 1, 7, bm, bn, 64, 2, ops.EPI_ALL_SCATTER, variant=variant)
+        elif epilogue == "store32":
+            out = shmem.zeros((M, N), dtype=torch.float32)
+            ops.gemm_launch(a, b, None, out, None, None, 0, 1, 7, bm, bn, 64, 2, ops.EPI_ALL_SCATTER, notify=False,
+                            variant=variant)
+        elif epilogue == "atomic32":
+            out = shmem.zeros((M, N), dtype=torch.float32)
+            ops.gemm_launch(a, b, None, out, None, None, 0, 1, 7, bm, bn, 64, 2, ops.EPI_ATOMIC_ADD, variant=variant)
+        else:
+            out = shmem.zeros((M, N), dtype=dtype)
+            partials, locks = split_workspace(shmem, 256, bm, bn)
+            assert total * 3 <= 256  # a program for every (tile, part) pair
+            ops.gemm_launch(a, b, None, out, flags, None, 0, 1, 256, bm, bn, 64, 2, ops.EPI_ALL_SCATTER,
+                            partials=partials, locks=locks, split_k=3, split_handover=ops.HANDOVER_SLICED,
+                            variant=variant)
+            torch.cuda.synchronize()
+            assert int(locks.abs().max().item()) == 0
+        torch.cuda.synchronize()
+        got[variant] = out.cpu().clone()
+        if epilogue in ("scatter16", "split_k"):
+            assert flags.cpu().tolist() == [1] * total
+    check_close(got[f4_variant].to(torch.float32), O.shard_gemm(A, B, None), f4_name)
+    width = torch.int16 if got[f4_variant].dtype == dtype else torch.int32
+    assert torch.equal(got[f4_variant].view(width), got[plain_variant].view(width)), f"{f4_name} vs {plain_name}"
+
+
 # --------------------------------------------------------------------------- split-K
 def split_workspace(shmem, grid, BM, BN):
     return (shmem.zeros((grid, BM * BN), dtype=torch.float32), shmem.zeros((grid,), dtype=torch.int32))
