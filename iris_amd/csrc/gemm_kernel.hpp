@@ -23,6 +23,12 @@
 //     The barrier that hands over the next stage sits inside a step's MFMA
 //     stream, so neither LDS latency nor the barrier is paid with idle
 //     matrix cores.
+//   * The four-wave tiles run with four more waves, one per SIMD, that only
+//     issue the stage loads and wait for them (GemmCfg::LW): a wave that is
+//     held up at the issue of a load multiplies nothing meanwhile, and with
+//     one wave per SIMD a K-step then costs fetch plus multiply instead of
+//     the longer of the two.  All waves run the same control flow and meet
+//     at the same barriers; only the work is told apart.
 //   * The epilogue transposes the accumulators through a wave-private LDS
 //     scratch so that global stores / atomics cover contiguous row segments.
 //     Stores are write-through at the flags' scope; once they have completed
