@@ -91,7 +91,7 @@ bool plan_few_rows(const iris_gemm_args& a, int op, bool dma_ok, Plan* plan) {
                   ((int64_t)SKINNY_ROWS * a.stride_am + a.K) * 2 < lim &&
                   ((int64_t)SKINNY_COLS * a.stride_bn + a.K) * 2 < lim;
   if (!ok) return false;
-  plan->skinny = gemm_skinny_kernel_for(a.ab_dtype, op, un);
+  plan->skinny = gemm_skinny_kernel_for(a.ab_dtype, op, un, a.M >= SKINNY_A_VIA_LDS_ROWS && a.K >= SKINNY_A_VIA_LDS_K);
   if (!plan->skinny) return false;
   plan->skinny_lds = skinny_lds_bytes(un);
   plan->skinny_grid = n_blocks;

@@ -34,10 +34,24 @@ constexpr int SKINNY_WAVES = 8;
 constexpr int SKINNY_THREADS = SKINNY_WAVES * 64;
 constexpr int SKINNY_RED_BYTES = SKINNY_WAVES * 64 * 16;  // the waves' partial accumulators
 constexpr int SKINNY_BLOCK_BYTES = 2048;                  // 16 rows of B x 64 k
-constexpr int skinny_lds_bytes(int un) { return SKINNY_RED_BYTES + SKINNY_WAVES * un * SKINNY_BLOCK_BYTES; }
+// a block of A per wave (the waves' partial accumulators take its place once the K range is done), then
+// every wave's UN blocks of B
+constexpr int SKINNY_A_BYTES = SKINNY_WAVES * SKINNY_BLOCK_BYTES;
+static_assert(SKINNY_RED_BYTES <= SKINNY_A_BYTES, "the partial accumulators reuse the blocks of A");
+constexpr int skinny_lds_bytes(int un) { return SKINNY_A_BYTES + SKINNY_WAVES * un * SKINNY_BLOCK_BYTES; }
+
+// From this many rows and this long a K on, A is fetched lanes-along-a-row
+// and passed through LDS.  Below, a load in operand layout only touches the
+// lanes of the rows that exist and is the cheaper way: [M,4096] x [4096,1376]
+// 6.8 against 7.3 us at one row, 7.4 both ways at four, 8.2 against 7.5 at
+// eight, 9.8 against 7.8 at sixteen; with K = 1376 (and 256 workgroups) the
+// pass through LDS never pays (16 rows: 6.6 against 6.7 us).
+constexpr int SKINNY_A_VIA_LDS_ROWS = 5;
+constexpr int SKINNY_A_VIA_LDS_K = 2048;
 
 // UN: K blocks (64 k each) whose fetches a wave has in flight together.
-template <int DT, int OP, int ODT, int UN>
+// A_LDS: how A reaches the MFMAs (see below).
+template <int DT, int OP, int ODT, int UN, bool A_LDS>
 __global__ __launch_bounds__(SKINNY_THREADS) __attribute__((amdgpu_waves_per_eu(2, UN == 8 ? 2 : UN == 4 ? 4 : 8))) void
 gemm_skinny_kernel(const GemmKArgs p) {
   constexpr bool ATOMIC = OP == OP_ATOMIC32 || OP == OP_ATOMIC16;
@@ -45,7 +59,7 @@ gemm_skinny_kernel(const GemmKArgs p) {
   using vec8 = typename Mfma<DT>::vec8;
   extern __shared__ __attribute__((aligned(1024))) char skinny_lds[];
   IRIS_LDS char* lds = (IRIS_LDS char*)skinny_lds;
-  // [SKINNY_WAVES][64] partial accumulators, then each wave's UN blocks of B
+  // each wave's block of A ([SKINNY_WAVES][64] partial accumulators at the end), then each wave's UN blocks of B
   IRIS_LDS f32x4* red = (IRIS_LDS f32x4*)lds;
 
   const int tid = threadIdx.x;
@@ -54,7 +68,8 @@ gemm_skinny_kernel(const GemmKArgs p) {
   const int lr = lane & 15, lq = lane >> 4;
   const int n0 = blockIdx.x * SKINNY_COLS;
   const int m0 = blockIdx.y * SKINNY_ROWS;
-  IRIS_LDS char* wb = lds + SKINNY_RED_BYTES + wave * (UN * SKINNY_BLOCK_BYTES);
+  IRIS_LDS char* wb = lds + SKINNY_A_BYTES + wave * (UN * SKINNY_BLOCK_BYTES);
+  IRIS_LDS char* wa = lds + wave * SKINNY_BLOCK_BYTES;
 
   // Rows past the edge of either operand lie past the end of its buffer
   // descriptor and read as zero; chunks past K are parked out of range.
@@ -69,15 +84,22 @@ gemm_skinny_kernel(const GemmKArgs p) {
   // chunk of the row it must bring there is (l%8) ^ (row/2 % 8).
   const int brow = lane >> 3;  // + 8j
   const int bchunk = (lane & 7) ^ ((brow >> 1) & 7);  // rows 8j + .. : (row/2)%8 = 4j + brow/2, and 4j flips bit 2
-  // A and the operand reads: lane l holds row l%16.  In K block kb, MFMA h
-  // (0, 1) takes k = kb*64 + (l/16)*16 + h*8 .. +7 at MFMA position
-  // (l/16)*8 .. +7: the same permutation of k for both operands.
+  // A_LDS: A comes in the same way, lanes along a row, but into registers: a
+  // load in operand layout (lane l holds row l%16) has neighbouring lanes in
+  // different rows, nothing for the memory pipeline to merge, and with 16 rows
+  // costs eight times what the same bytes of B cost (2.5 against 0.3 us).  A
+  // block of A then goes through a 2 KiB region of the wave, laid out like a
+  // block of B, on its way to the MFMAs.  With very few rows the load in
+  // operand layout is the cheaper one (!A_LDS).
+  // The operand reads: lane l holds row l%16.  In K block kb, MFMA h (0, 1)
+  // takes k = kb*64 + (l/16)*16 + h*8 .. +7 at MFMA position (l/16)*8 .. +7:
+  // the same permutation of k for both operands.
   const uint32_t oa = (uint32_t)(((int64_t)lr * p.sam + lq * 16) * 2);
   const int nb = (p.K + 63) / 64;
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int b0 = wave; b0 < nb; b0 += SKINNY_WAVES * UN) {
-    vec8 fa[UN][2];
+    u32x4 va[UN][2];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int kb = b0 + SKINNY_WAVES * u;
@@ -90,10 +112,16 @@ gemm_skinny_kernel(const GemmKArgs p) {
                                                  ok ? (int)off : (int)0x80000000, 0, 0, 0);
       }
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const bool ok = kb < nb && kb * 64 + lq * 16 + h * 8 < p.K;
-        fa[u][h] = __builtin_bit_cast(
-            vec8, __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? (int)(oa + kb * 128 + h * 16) : (int)0x80000000, 0, 0));
+      for (int j = 0; j < 2; ++j) {
+        if constexpr (A_LDS) {
+          const int ch = bchunk ^ (j << 2);
+          const bool ok = kb < nb && kb * 64 + ch * 8 < p.K;
+          const uint32_t off = (uint32_t)(((int64_t)(brow + 8 * j) * p.sam) * 2 + kb * 128 + ch * 16);
+          va[u][j] = __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? (int)off : (int)0x80000000, 0, 0);
+        } else {  // j is the MFMA (h) the 16 bytes are for
+          const bool ok = kb < nb && kb * 64 + lq * 16 + j * 8 < p.K;
+          va[u][j] = __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? (int)(oa + kb * 128 + j * 16) : (int)0x80000000, 0, 0);
+        }
       }
     }
     // every fetch is on its way; B has landed in this wave's own region once
@@ -101,13 +129,25 @@ gemm_skinny_kernel(const GemmKArgs p) {
     IRIS_WAIT_VMCNT(0);
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int u = 0; u < UN; ++u)
+    for (int u = 0; u < UN; ++u) {
+      // (the wave's LDS operations execute in order: these writes land after
+      // the previous block's reads and before this block's)
+      if constexpr (A_LDS) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) *reinterpret_cast<IRIS_LDS u32x4*>(wa + j * 1024 + lane * 16) = va[u][j];
+      }
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const int pc = (lq * 2 + h) ^ ((lr >> 1) & 7);
         const vec8 fb = *reinterpret_cast<const IRIS_LDS vec8*>(wb + u * SKINNY_BLOCK_BYTES + lr * 128 + pc * 16);
-        acc = Mfma<DT>::run(fb, fa[u][h], acc);
+        vec8 fa;
+        if constexpr (A_LDS)
+          fa = *reinterpret_cast<const IRIS_LDS vec8*>(wa + lr * 128 + pc * 16);
+        else
+          fa = __builtin_bit_cast(vec8, va[u][h]);
+        acc = Mfma<DT>::run(fb, fa, acc);
       }
+    }
     // the reads above have returned before the next round overwrites the region
     IRIS_WAIT_LGKMCNT0();
     asm volatile("" ::: "memory");
@@ -115,6 +155,7 @@ gemm_skinny_kernel(const GemmKArgs p) {
 
   // acc: row m = l%16 of C, columns n0 + 4*(l/16) .. +3 (operands swapped, as
   // in the persistent kernel)
+  if constexpr (A_LDS) __syncthreads();  // every wave is done with its block of A: the region becomes `red`
   red[wave * 64 + lane] = acc;
   __syncthreads();
 
@@ -195,7 +236,7 @@ gemm_skinny_kernel(const GemmKArgs p) {
   }
 }
 
-// The kernel for (operand type, store op, blocks in flight), or null.
-GemmKernelFn gemm_skinny_kernel_for(int dt, int op, int un);
+// The kernel for (operand type, store op, blocks in flight, A through LDS), or null.
+GemmKernelFn gemm_skinny_kernel_for(int dt, int op, int un, bool a_lds);
 
 }  // namespace iris_amd

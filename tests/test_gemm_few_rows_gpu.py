@@ -38,6 +38,10 @@ CASES = [
     (17, 1376, 4096, 64, 64, 4, torch.bfloat16),    # two blocks of rows, the second with one row
     (32, 4096, 1376, 32, 128, 6, torch.bfloat16),
     (20, 50, 72, 32, 16, 2, torch.float16),         # one block of columns per flag, two of rows
+    # (from five rows and K = 2048 on, A is fetched along its rows and passed through LDS)
+    (9, 200, 2120, 64, 64, 2, torch.float16),       # ... with a K tail of 8 and a ragged last block of columns
+    (32, 512, 2048, 32, 64, 2, torch.bfloat16),     # ... two blocks of rows
+    (4, 1376, 4096, 64, 64, 4, torch.bfloat16),     # (four rows: still fetched in operand layout)
 ]
 
 
