@@ -103,8 +103,9 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 #define IRIS_STATUS_SPIN_TIMEOUT 1 /* a flag wait gave up; that tile was not reduced */
 
 /* Special values of iris_gemm_args.variant.  A launch with at most 32 rows of
- * A whose operands are K-contiguous normally takes a kernel of its own that
- * streams B (one workgroup per 16 rows x 16 columns of C, all fetches in flight);
+ * A (64 when K >= 2048) whose operands are K-contiguous normally takes a kernel
+ * of its own that streams B (one workgroup per 16 or 32 rows x 16 columns of C,
+ * all fetches in flight);
  * FEW_ROWS insists on it (hipErrorInvalidValue when the launch does not
  * qualify), PERSISTENT keeps the default choice among the persistent kernels.
  * The reference has one Triton kernel for every M (gemm_all_scatter.py:95). */
@@ -221,7 +222,7 @@ int iris_gemm_kernel_info(const iris_gemm_args* args, int* n_regs, int* n_spills
 int iris_gemm_split_k(const iris_gemm_args* args, int* split_k);
 
 /* Name of the kernel `iris_gemm_launch` would run for `args` ("" when there is
- * no GEMM work): a tuning variant's name, or "few_rows_16xN". */
+ * no GEMM work): a tuning variant's name, or "few_rows_16xN" / "few_rows_32xN". */
 int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t len);
 
 /* Name of tuning variant `variant` (1-based) of the kernel list used for

@@ -63,6 +63,94 @@ def test_scatter_single_rank(shmem, M, N, K, BM, BN, G, dtype):
         assert not locks.any()
 
 
+MID = "few_rows_32xN"
+MID_CASES = [
+    # M, N, K, BLK_M, BLK_N, G, dtype: 33 to 64 rows of a K of 2048 or more, one round of workgroups
+    (64, 1376, 4096, 64, 64, 4, torch.bfloat16),    # decoder gate/up at 64 tokens: 2 x 86 workgroups
+    (33, 1376, 4096, 256, 64, 4, torch.bfloat16),   # the second block of rows holds one row
+    (48, 200, 2120, 64, 16, 2, torch.float16),      # K tail of 8, ragged last block of columns, a workgroup a flag
+    (50, 272, 9000, 64, 48, 3, torch.bfloat16),     # K range that takes a wave two rounds of fetches
+]
+
+
+@pytest.mark.parametrize("M,N,K,BM,BN,G,dtype", MID_CASES)
+def test_scatter_33_to_64_rows(shmem, M, N, K, BM, BN, G, dtype):
+    """32 rows x 16 columns a workgroup: the same exchange, with two
+    accumulator blocks a wave summed block by block before the stores."""
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.full((M, N), 7, dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total + 3,), dtype=torch.int32)
+    locks = shmem.zeros((256,), dtype=torch.int32)
+    for launch in (1, 2):
+        cg.fill_(7)
+        assert scatter(shmem, a, b, cg, flags, 0, 1, BM, BN, G, locks=locks) == MID
+        torch.cuda.synchronize()
+        check_close(cg, O.shard_gemm(A, B, dtype), f"launch {launch}")
+        assert flags.cpu().tolist() == [launch] * total + [0, 0, 0]
+        assert not locks.any()
+
+
+def test_33_to_64_rows_other_epilogues_and_the_launcher_choice(shmem):
+    """fp32 partial with the one-shot signal on 4 virtual ranks, atomic add; and
+    when the launch stays with the persistent kernels."""
+    ws, M, N, K, dtype = 4, 40, 384, 4 * 2048, torch.bfloat16
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    shards = O.k_shards(A, B, ws)
+    ah, bh = to_heap(shmem, A), to_heap(shmem, B)
+    kk = K // ws
+    part = shmem.zeros((M, N), dtype=torch.float32)
+    out = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(N, 128)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    locks = shmem.zeros((256,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+    for r in range(ws):
+        for t in (part, out, flags, locks):
+            shmem.on_rank(t, r).zero_()
+    for r in range(ws):
+        args = (ah[:, r * kk:(r + 1) * kk], bh[r * kk:(r + 1) * kk, :], shmem.on_rank(part, r), shmem.on_rank(out, r),
+                shmem.on_rank(flags, r), hb, r, ws, 256, 64, 128, 64, 6, ops.EPI_ONE_SHOT)
+        kw = dict(phase=ops.PHASE_PRODUCE, locks=shmem.on_rank(locks, r))
+        assert ops.gemm_plan_name(*args, **kw) == MID
+        ops.gemm_launch(*args, **kw)
+    torch.cuda.synchronize()
+    for r in range(ws):
+        check_close(shmem.on_rank(part, r), O.shard_gemm(*shards[r], torch.float32), f"partial {r}")
+        assert shmem.on_rank(flags, r).cpu().tolist() == [ws - 1] * total
+        assert not shmem.on_rank(locks, r).any()
+    # atomic accumulate of the four K shards into one fp32 C
+    c32 = shmem.zeros((M, N), dtype=torch.float32)
+    for r in range(ws):
+        args = (ah[:, r * kk:(r + 1) * kk], bh[r * kk:(r + 1) * kk, :], None, c32, None, None, 0, 1, 256, 64, 128, 64, 6,
+                ops.EPI_ATOMIC_ADD)
+        assert ops.gemm_plan_name(*args) == MID
+        ops.gemm_launch(*args)
+    torch.cuda.synchronize()
+    check_close(c32, O.atomics_all_reduce(shards))
+    # the persistent kernels keep: a short K, more rows, a logical tile that does not cover the rows, more
+    # workgroups than CUs, the caller's insistence
+    a1 = ah[:, :kk]
+    b1 = bh[:kk, :]
+    cg = shmem.zeros((M, N), dtype=dtype)
+    many_flags = shmem.zeros((1024,), dtype=torch.int32)
+
+    def plan(a_, b_, cg_, BM, BN, **kw):
+        return ops.gemm_plan_name(a_, b_, None, cg_, many_flags, None, 0, 1, 256, BM, BN, 64, 4, ops.EPI_ALL_SCATTER,
+                                  locks=locks, **kw)
+
+    assert plan(a1, b1, cg, 64, 128) == MID
+    assert plan(a1[:, :1024], b1[:1024, :], cg, 64, 128) != MID
+    assert plan(a1, b1, cg, 32, 128) != MID
+    assert plan(a1, b1, cg, 64, 128, variant=ops.VARIANT_PERSISTENT) != MID
+    A2, B2 = make_ab(65, 4096, 2048, dtype)
+    a2, b2 = to_heap(shmem, A2), to_heap(shmem, B2)
+    cg2 = shmem.zeros((65, 4096), dtype=dtype)
+    assert plan(a2, b2, cg2, 128, 128) != MID                    # more than 64 rows
+    assert plan(a2[:64], b2, cg2[:64], 64, 128) != MID            # 2 x 256 workgroups: more than one round
+
+
 def test_strided_operands_and_output(shmem):
     """K-shard views (leading dimensions > K) and an output that is a column
     block of a wider matrix."""

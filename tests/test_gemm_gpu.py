@@ -576,20 +576,20 @@ def test_split_k_all_scatter(shmem, M, N, K, BM, BN, split_k, dtype):
 
 def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
     dtype = torch.bfloat16
-    A, B = make_ab(40, 1376, 4096, dtype)  # (up to 16 rows would go to the few-rows kernel)
+    A, B = make_ab(72, 1376, 4096, dtype)  # (up to 64 rows would go to the few-rows kernel)
     a, b = to_heap(shmem, A), to_heap(shmem, B)
-    cg = shmem.zeros((40, 1376), dtype=dtype)
-    flags = shmem.zeros((32,), dtype=torch.int32)
+    cg = shmem.zeros((72, 1376), dtype=dtype)
+    flags = shmem.zeros((64,), dtype=torch.int32)
     partials, locks = split_workspace(shmem, 256, 64, 64)
     common = (a, b, None, cg, flags, None, 0, 1, 256, 64, 64, 64, 4, ops.EPI_ALL_SCATTER)
-    # 22 tiles on 256 programs, 64 K-steps: 11 parts each
-    assert ops.gemm_split_k(*common, partials=partials, locks=locks) == 11
+    # 44 tiles on 256 programs, K = 4096: 5 parts each
+    assert ops.gemm_split_k(*common, partials=partials, locks=locks) == 5
     assert ops.gemm_split_k(*common) == 1                                    # no workspace
     assert ops.gemm_split_k(*common, partials=partials, locks=locks, split_k=1) == 1
     ops.gemm_launch(*common, partials=partials, locks=locks)
     torch.cuda.synchronize()
     check_close(cg, O.shard_gemm(A, B, dtype))
-    assert flags.cpu().tolist()[:22] == [1] * 22 and int(locks.abs().max().item()) == 0
+    assert flags.cpu().tolist()[:44] == [1] * 44 and int(locks.abs().max().item()) == 0
     # enough tiles to fill the programs: unsplit
     A2, B2 = make_ab(1024, 1024, 512, dtype)
     a2, b2 = to_heap(shmem, A2), to_heap(shmem, B2)
@@ -601,7 +601,7 @@ def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
     with pytest.raises(ValueError):
         ops.gemm_launch(*common, split_k=4)                                  # no workspace
     with pytest.raises(ValueError):
-        ops.gemm_launch(*common, partials=partials, locks=locks, split_k=16)  # 22 * 16 pairs > 256 programs
+        ops.gemm_launch(*common, partials=partials, locks=locks, split_k=8)   # 44 * 8 pairs > 256 programs
     # the 128-accumulator tiles split too, with the sliced hand-over only
     big = shmem.zeros((256, 256 * 256), dtype=torch.float32)
     with pytest.raises(ValueError):
