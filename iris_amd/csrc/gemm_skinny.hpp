@@ -1,4 +1,4 @@
-// Shard GEMM for a few rows of A (decode-time batches, 16 rows a workgroup): C[M,N] = A[M,K] B[K,N]
+// Shard GEMM for a few rows of A (decode-time batches, 16 or 32 rows a workgroup): C[M,N] = A[M,K] B[K,N]
 // with the epilogues of the persistent kernel (gemm_all_scatter.py:209-251,
 // gemm_atomics_all_reduce.py:236-248, gemm_one_shot_all_reduce.py:197-218).
 //
@@ -13,9 +13,12 @@
 //     of a fetch in MFMA operand layout, 16 rows x 64 bytes), into a region of
 //     LDS private to the wave, 16-byte chunks XOR-ed by the row so that the
 //     operand reads are conflict-free;
-//   * A, at most 16 rows that every workgroup reads and L2 holds, goes
-//     straight into registers in operand layout.
-// The eight partial 16x16 accumulators meet in LDS; wave w then stores the
+//   * A, rows that every workgroup reads and L2 holds, goes into registers:
+//     straight in operand layout when there are very few of them, otherwise
+//     lanes along a row like B, each block passing through 2 KiB of LDS on
+//     its way to the MFMAs (a load in operand layout has neighbouring lanes
+//     in different rows and merges nothing).
+// The waves' partial 16x16 accumulators meet in LDS; wave w then stores the
 // sum on destination rank w, w+8, ...
 //
 // A logical tile (BLOCK_SIZE_M x BLOCK_SIZE_N, one flag; BLOCK_SIZE_M covers
