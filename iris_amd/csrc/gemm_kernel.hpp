@@ -1255,7 +1255,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
     Frags<Cfg> fr;
     if (total_steps > 0) {
       if (fetcher) {
-        l_it = decode_item<Cfg, SPLIT>(p, sr, pid, 0);
+        l_it = c_it;  // (item 0, decoded above for the compute cursor)
         const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, 0, nk);
         l_k = kr.k_begin;
         l_kend = kr.k_end;
