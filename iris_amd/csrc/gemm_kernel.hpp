@@ -171,7 +171,8 @@ struct GemmCfg {
   static_assert((CM * CPR) % (NL * 64) == 0 && (CN * CPR) % (NL * 64) == 0, "slab must split evenly over lanes");
   static_assert(LW == 0 || (DMA && NW + LW <= 8), "fetching waves: LDS-DMA tiles of at most eight waves in all");
   static_assert(A_LOADS >= 1 && B_LOADS >= 1, "too many waves for this slab");
-  static_assert((S & (S - 1)) == 0 && S >= 1, "ring depth must be a power of two");
+  static constexpr bool S_POW2 = (S & (S - 1)) == 0;  // (else the ring slot is counted along instead of masked out of g)
+  static_assert(S >= 1, "ring depth");
   static_assert(!DMA || S >= 2, "the DMA ring needs a stage being read and one in flight");
   static_assert(L * (S - 1) <= 63, "vmcnt immediate");
   static_assert(IM * IN * 4 <= 128, "accumulators of a wave tile: at most 128 registers");
@@ -1288,10 +1289,20 @@ gemm_persistent_kernel(const GemmKArgs p) {
     // g+S, a few DMA loads per block.  The program's very last step hands over
     // too; what it fetches is never used (loads past the last step fetch
     // nothing).
+    int ring_slot = 0;  // slot of the step about to run (rings whose depth is no power of two)
     auto step = [&](int g, auto first_tag, auto par_tag) __attribute__((always_inline)) {
       constexpr bool FIRST = decltype(first_tag)::value;
       constexpr int PAR = decltype(par_tag)::value;
-      const IRIS_LDS char* stage = lds + (g & (Cfg::S - 1)) * Cfg::STAGE;
+      int slot_g, slot_n;  // ring slots of steps g and g+1
+      if constexpr (Cfg::S_POW2) {
+        slot_g = g & (Cfg::S - 1);
+        slot_n = (g + 1) & (Cfg::S - 1);
+      } else {
+        slot_g = ring_slot;
+        slot_n = ring_slot + 1 == Cfg::S ? 0 : ring_slot + 1;
+        ring_slot = slot_n;
+      }
+      const IRIS_LDS char* stage = lds + slot_g * Cfg::STAGE;
       if (worker) {
 #pragma unroll
         for (int kk = 0; kk < Cfg::KSUB - 1; ++kk) {
@@ -1347,10 +1358,10 @@ gemm_persistent_kernel(const GemmKArgs p) {
             pending_skip = 0;
           }
         }
-        const IRIS_LDS char* nstage = lds + ((g + 1) & (Cfg::S - 1)) * Cfg::STAGE;
+        const IRIS_LDS char* nstage = lds + slot_n * Cfg::STAGE;
         const IRIS_LDS char* sA = nstage + a_row_off + xoff[0];
         const IRIS_LDS char* sB = nstage + Cfg::A_BYTES + b_row_off + xoff[0];
-        IRIS_LDS char* rstage = lds + (g & (Cfg::S - 1)) * Cfg::STAGE;
+        IRIS_LDS char* rstage = lds + slot_g * Cfg::STAGE;
         if (worker) {
           fr.a[0] = load_a<Cfg>(sA, 0);
           load_b_share<Cfg>(sB, 0, fr.b[cb ^ 1]);

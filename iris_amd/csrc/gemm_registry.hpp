@@ -62,16 +62,19 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 //
 // The four-wave tiles come twice: with one fetching wave per SIMD beside the
 // multiplying one (`_f4`: a K-step then costs the longer of fetch and multiply
-// instead of their sum; [2048,4096] x [4096,1376] in 128 x 128 tiles 48 -> 40 us),
-// and plain, which the launcher takes where the first loses: with the reduce
-// inside the program (no such build), for a split launch of a 128-accumulator
-// tile (its fetch state spills there), and for two programs per CU.
+// instead of their sum; [2048,4096] x [4096,1376] in 128 x 128 tiles 48 -> 40 us)
+// and as deep a ring as LDS holds, since a fetching wave cannot refill the
+// stage that is being multiplied (256 x 64 tiles in three stages instead of
+// two: 57 -> 42 us on the same shape); and plain, which the launcher takes
+// where the first loses: with the reduce inside the program (no such build),
+// for a split launch of a 128-accumulator tile (its fetch state spills there),
+// and for two programs per CU.
 #define IRIS_GEMM_VARIANTS(X, DT, OP)                                     \
   X(DT, OP, 256, 256, 64, 2, 4, 2, true, 0, 1, "256x256x64_w2x4_s2")         \
-  X(DT, OP, 256, 128, 64, 2, 2, 2, true, 4, 1, "256x128x64_w2x2_s2_f4")      \
-  X(DT, OP, 128, 256, 64, 1, 4, 2, true, 4, 1, "128x256x64_w1x4_s2_f4")      \
+  X(DT, OP, 256, 128, 64, 2, 2, 3, true, 4, 1, "256x128x64_w2x2_s3_f4")      \
+  X(DT, OP, 128, 256, 64, 1, 4, 3, true, 4, 1, "128x256x64_w1x4_s3_f4")      \
   X(DT, OP, 128, 128, 64, 2, 2, 4, true, 4, 1, "128x128x64_w2x2_s4_f4")      \
-  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")        \
+  X(DT, OP, 256, 64, 64, 4, 1, 3, true, 4, 1, "256x64x64_w4x1_s3_f4")        \
   X(DT, OP, 128, 64, 64, 2, 2, 4, true, 4, 1, "128x64x64_w2x2_s4_f4")        \
   X(DT, OP, 64, 128, 64, 2, 2, 4, true, 4, 1, "64x128x64_w2x2_s4_f4")        \
   X(DT, OP, 64, 64, 128, 2, 2, 4, true, 4, 1, "64x64x128_w2x2_s4_f4")        \
@@ -89,7 +92,8 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   X(DT, OP, 256, 128, 64, 2, 4, 2, true, 0, 1, "256x128x64_w2x4_s2")         \
   X(DT, OP, 128, 256, 64, 2, 4, 2, true, 0, 1, "128x256x64_w2x4_s2")         \
   X(DT, OP, 128, 128, 32, 2, 2, 4, true, 0, 0, "128x128x32_w2x2_s4")         \
-  X(DT, OP, 64, 64, 64, 2, 2, 4, true, 4, 1, "64x64x64_w2x2_s4_f4")
+  X(DT, OP, 64, 64, 64, 2, 2, 4, true, 4, 1, "64x64x64_w2x2_s4_f4")          \
+  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")
 
 #define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, SPLIT, NAME) \
   make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP>(NAME),
