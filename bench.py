@@ -612,6 +612,14 @@ def main():
                                      "roofline": {"bound": "mfma", "achieved": round(cold_tflops, 2),
                                                   "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                                   "frac": round(cold_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}}
+        if not args.no_context:
+            # the vendor library's GEMM on the same operands under the same protocol (no flags)
+            lib_out = torch.empty((M, N), dtype=dtype, device="cuda")
+            lib_cold_ms = iris_amd.do_bench(lambda: torch.matmul(a, b, out=lib_out), shmem.barrier, lambda: None,
+                                            n_warmup=10, n_repeat=50)
+            result["gemm_cold_cache"]["library_ms"] = round(lib_cold_ms, 5)
+            result["gemm_cold_cache"]["library_tflops"] = round(flops / (lib_cold_ms * 1e-3) / 1e12, 2)
+            del lib_out
 
     if not args.no_reduce:
         # reduce phase: 8 fp32 partials [8192,8192] (one per virtual rank) -> bf16
