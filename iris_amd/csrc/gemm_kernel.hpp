@@ -69,6 +69,9 @@ struct GemmKArgs {
   TileDivs tile_divs;
   FastDiv div_subs, div_sub_n;  // sub_m * sub_n, sub_n
   FastDiv div_split, div_nk;    // split_k; K-steps of a tile (stream-K runs)
+  // > 1: the launch's tiles (BN, num_pid_n, tile ids above) are `merge_n` of the caller's tiles side by side;
+  // the flags stay the caller's, one per tile of width BN / merge_n, numbered over flag_num_pid_n columns
+  int merge_n, flag_num_pid_n;
   int dest_all;      // write `out` on every rank's heap (else on this rank only)
   int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
   int sys;           // flag atomics at system scope (else agent)
@@ -678,13 +681,24 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
 // vector load and the increments leave together (one thread walking the ranks
 // waits for a scalar load per rank: 0.8 us for eight).
 __device__ inline void publish_tile(const GemmKArgs& p, int tile_id, int lane) {
-  IRIS_GLOBAL int32_t* own = (IRIS_GLOBAL int32_t*)(p.flags + tile_id);
-  for (int r = lane; r < p.ws; r += 64) {
-    if (p.flag_mode == 2 && r == p.cur_rank) continue;
-    IRIS_GLOBAL int32_t* f = own;
-    if (r != p.cur_rank && p.heap_bases != nullptr)
-      f = translate(p.flags + tile_id, p.heap_bases[p.cur_rank], p.heap_bases[r]);
-    flag_add_relaxed(f, 1, p.sys != 0);
+  // the caller's tiles the launch's tile covers: itself, or merge_n in a row
+  int first = tile_id, count = 1, pid_m = 0, pn0 = 0;
+  if (p.merge_n > 1) {
+    const TileCoord t = tile_map_fast(tile_id, p.num_pid_m, p.num_pid_n, p.G, p.tile_divs);
+    pid_m = t.pid_m;
+    pn0 = t.pid_n * p.merge_n;
+    count = min(p.merge_n, p.flag_num_pid_n - pn0);
+  }
+  for (int j = 0; j < count; ++j) {
+    if (p.merge_n > 1) first = tile_id_of(pid_m, pn0 + j, p.num_pid_m, p.flag_num_pid_n, p.G);
+    IRIS_GLOBAL int32_t* own = (IRIS_GLOBAL int32_t*)(p.flags + first);
+    for (int r = lane; r < p.ws; r += 64) {
+      if (p.flag_mode == 2 && r == p.cur_rank) continue;
+      IRIS_GLOBAL int32_t* f = own;
+      if (r != p.cur_rank && p.heap_bases != nullptr)
+        f = translate(p.flags + first, p.heap_bases[p.cur_rank], p.heap_bases[r]);
+      flag_add_relaxed(f, 1, p.sys != 0);
+    }
   }
 }
 

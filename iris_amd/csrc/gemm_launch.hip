@@ -211,7 +211,49 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
 // Validate `a` and build the launch plan.  Returns hipSuccess,
 // hipErrorInvalidValue, or a pseudo-success with entry == nullptr when there
 // is no GEMM work to do.
+hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan);
+
+// The plan of a launch.  A caller's tile that is 256 rows tall and narrow (the reference scripts' 256 x 64)
+// makes a large GEMM wait for its operands: every K-step fetches 256 rows of A for 64 columns' worth of work.
+// Where there are enough of them, the launch computes two or four of the caller's tiles, side by side, as one
+// 256 x 128 or 256 x 256 tile and raises each one's flag: tile ids and flags are the caller's, which program
+// computes a tile was never observable ([8192,8192] x [8192,1024] in 256 x 64 tiles: 739-762 -> 902 TFLOP/s
+// over the eight ranks of the reference's 07 benchmark).
 hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
+  int merge = 1;
+  const bool plain = a.variant == 0 && a.split_k == 0 && !a.mm_begin_timestamp && !a.mm_end_timestamp &&
+                     !(a.epilogue == IRIS_EPI_ONE_SHOT && a.phase == IRIS_PHASE_FUSED) &&
+                     a.epilogue != IRIS_EPI_ATOMIC_ADD && a.num_sms > 0 && a.block_m == 256 &&
+                     (a.block_n == 64 || a.block_n == 128) && a.M >= 256;
+  if (plain) {
+    const int64_t tiles = (int64_t)((a.M + 255) / 256) * ((a.N + a.block_n - 1) / a.block_n);
+    const int up_to = 256 / a.block_n;  // 4 or 2
+    if (tiles >= (int64_t)up_to * a.num_sms)
+      merge = up_to;
+    else if (up_to == 4 && tiles >= 2 * (int64_t)a.num_sms)
+      merge = 2;
+  }
+  if (merge > 1) {
+    iris_gemm_args b = a;
+    b.block_n = a.block_n * merge;
+    Plan merged;
+    const hipError_t err = make_plan_body(b, &merged);
+    // (only the persistent kernels, unsplit, publish merged tiles)
+    if (err == hipSuccess && merged.entry && !merged.skinny && merged.k.split_k == 1 && !merged.k.stream_k &&
+        !merged.in_program) {
+      *plan = merged;
+      plan->k.merge_n = merge;
+      plan->k.flag_num_pid_n = (a.N + a.block_n - 1) / a.block_n;
+      return hipSuccess;
+    }
+  }
+  const hipError_t err = make_plan_body(a, plan);
+  plan->k.merge_n = 1;
+  plan->k.flag_num_pid_n = plan->k.num_pid_n;
+  return err;
+}
+
+hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan) {
   if (a.M < 0 || a.N < 0 || a.K < 0) return hipErrorInvalidValue;
   if (a.block_m <= 0 || a.block_n <= 0 || a.group_size_m <= 0) return hipErrorInvalidValue;
   if (a.num_sms <= 0 || a.num_xcds <= 0 || (a.num_sms % a.num_xcds) != 0) return hipErrorInvalidValue;
@@ -659,11 +701,14 @@ extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t
   hipError_t err = make_plan(*args, &plan);
   if (err != hipSuccess) return err;
   const char* few = plan.skinny_rb == 2 ? "few_rows_32xN" : "few_rows_16xN";
-  std::snprintf(buf, len, "%s%s", plan.skinny ? few : plan.entry ? plan.entry->name : "",
+  std::snprintf(buf, len, "%s%s%s", plan.skinny ? few : plan.entry ? plan.entry->name : "",
                 plan.entry && plan.k.stream_k                   ? "+stream_k"
                 : plan.entry && plan.in_program                 ? "+reduce"
                 : plan.entry && plan.k.num_sms > args->num_sms ? "+two_per_cu"
-                                                                : "");
+                                                                : "",
+                plan.entry && plan.k.merge_n == 2   ? "+two_tiles_each"
+                : plan.entry && plan.k.merge_n == 4 ? "+four_tiles_each"
+                                                    : "");
   return hipSuccess;
 }
 

@@ -522,6 +522,76 @@ def test_build_with_fetching_waves_is_bit_identical_to_the_plain_build(shmem, ep
     assert torch.equal(got[f4_variant].view(width), got[plain_variant].view(width)), f"{f4_name} vs {plain_name}"
 
 
+@pytest.mark.parametrize("M,N,K,BN,grid,ws,suffix", [
+    (1024, 640, 256, 64, 2, 1, "+four_tiles_each"),    # 4 x 10 tiles: the last merged tile of a row covers two
+    (1024, 640, 256, 64, 16, 2, "+two_tiles_each"),    # 40 tiles on 16 programs: pairs; flags on both ranks
+    (520, 392, 328, 128, 3, 1, "+two_tiles_each"),     # 3 x 4 tiles of 256 x 128, ragged edges
+    (1024, 640, 256, 64, 32, 1, ""),                   # too few tiles for the programs: as the caller cut them
+])
+def test_narrow_tall_tiles_are_computed_several_at_a_time(shmem, M, N, K, BN, grid, ws, suffix):
+    """A caller's 256 x 64 (or 256 x 128) tiles, where there are enough of them,
+    are computed two or four side by side as one tile; every one of the
+    caller's flags is raised exactly once, on every rank, and nothing else."""
+    dtype = torch.bfloat16
+    A, B = make_ab(M, N * ws, K, dtype)
+    shards = O.n_shards(A, B, ws)
+    a = to_heap(shmem, A)
+    bs = [to_heap(shmem, sb) for _, sb in shards]
+    cg = shmem.zeros((M, N * ws), dtype=dtype)
+    total = ops.cdiv(M, 256) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total + 5,), dtype=torch.int32)
+    hb = shmem.get_heap_bases() if ws > 1 else None
+    for r in range(ws):
+        for t in (cg, flags):
+            shmem.on_rank(t, r).zero_()
+    for r in range(ws):
+        args = (a, bs[r], None, shmem.on_rank(cg, r), shmem.on_rank(flags, r), hb, r, ws, grid, 256, BN, 64, 4,
+                ops.EPI_ALL_SCATTER)
+        name = ops.gemm_plan_name(*args)
+        assert name.endswith(suffix) and (suffix or "tiles_each" not in name), name
+        ops.gemm_launch(*args)
+    torch.cuda.synchronize()
+    want = O.all_scatter(shards, dtype)
+    for r in range(ws):
+        check_close(shmem.on_rank(cg, r), want, f"rank {r}")
+        assert shmem.on_rank(flags, r).cpu().tolist() == [ws] * total + [0] * 5
+
+
+def test_merged_tiles_with_the_one_shot_producer_and_reduce(shmem):
+    """ONE_SHOT over 2 virtual ranks with the reference's default 256 x 64
+    tile: the producers compute four tiles at a time and signal each tile's
+    flag on the other rank; the reduce waits per tile of the caller's."""
+    ws, M, N, K, dtype = 2, 512, 512, 2 * 192, torch.bfloat16
+    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    shards = O.k_shards(A, B, ws)
+    ah, bh = to_heap(shmem, A), to_heap(shmem, B)
+    kk = K // ws
+    part = shmem.zeros((M, N), dtype=torch.float32)
+    out = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, 256) * ops.cdiv(N, 64)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+    for r in range(ws):
+        for t in (part, out, flags):
+            shmem.on_rank(t, r).zero_()
+    for r in range(ws):
+        args = (ah[:, r * kk:(r + 1) * kk], bh[r * kk:(r + 1) * kk, :], shmem.on_rank(part, r), shmem.on_rank(out, r),
+                shmem.on_rank(flags, r), hb, r, ws, 4, 256, 64, 64, 6, ops.EPI_ONE_SHOT)
+        assert ops.gemm_plan_name(*args, phase=ops.PHASE_PRODUCE).endswith("+four_tiles_each")
+        ops.gemm_launch(*args, phase=ops.PHASE_PRODUCE)
+    torch.cuda.synchronize()
+    for r in range(ws):
+        assert shmem.on_rank(flags, r).cpu().tolist() == [ws - 1] * total
+    for r in range(ws):
+        ops.one_shot_reduce(shmem.on_rank(part, r), shmem.on_rank(out, r), shmem.on_rank(flags, r), hb, r, ws, 256, 64,
+                            6)
+    torch.cuda.synchronize()
+    want = O.one_shot_all_reduce(shards, torch.float32, dtype)
+    for r in range(ws):
+        check_close(shmem.on_rank(out, r), want, f"reduced on rank {r}")
+        assert not shmem.on_rank(flags, r).any()
+
+
 # --------------------------------------------------------------------------- split-K
 def split_workspace(shmem, grid, BM, BN):
     return (shmem.zeros((grid, BM * BN), dtype=torch.float32), shmem.zeros((grid,), dtype=torch.int32))
