@@ -224,9 +224,9 @@ int iris_gemm_split_k(const iris_gemm_args* args, int* split_k);
 /* Name of the kernel `iris_gemm_launch` would run for `args` ("" when there is
  * no GEMM work): a tuning variant's name, or "few_rows_16xN" / "few_rows_32xN",
  * followed by "+stream_k", "+reduce" (the in-program reduce) or "+two_per_cu"
- * (two programs a CU), and by "+two_tiles_each" / "+four_tiles_each" where the
- * launch computes that many of the caller's 256-row tiles side by side as one
- * (each tile keeps its own id and flag). */
+ * (two programs a CU), and by "+two_tiles_each" / "+four_tiles_each" /
+ * "+eight_tiles_each" where the launch computes a block of that many of the
+ * caller's tiles as one (each tile keeps its own id and flag). */
 int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t len);
 
 /* Name of tuning variant `variant` (1-based) of the kernel list used for

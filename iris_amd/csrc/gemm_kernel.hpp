@@ -69,9 +69,10 @@ struct GemmKArgs {
   TileDivs tile_divs;
   FastDiv div_subs, div_sub_n;  // sub_m * sub_n, sub_n
   FastDiv div_split, div_nk;    // split_k; K-steps of a tile (stream-K runs)
-  // > 1: the launch's tiles (BN, num_pid_n, tile ids above) are `merge_n` of the caller's tiles side by side;
-  // the flags stay the caller's, one per tile of width BN / merge_n, numbered over flag_num_pid_n columns
-  int merge_n, flag_num_pid_n;
+  // merge_m * merge_n > 1: the launch's tiles (BM, BN, num_pid_m, num_pid_n, tile ids above) are merge_m x
+  // merge_n of the caller's tiles; the flags stay the caller's, one per tile of BM / merge_m x BN / merge_n,
+  // numbered over flag_num_pid_m x flag_num_pid_n tiles
+  int merge_m, merge_n, flag_num_pid_m, flag_num_pid_n;
   int dest_all;      // write `out` on every rank's heap (else on this rank only)
   int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
   int sys;           // flag atomics at system scope (else agent)
@@ -681,25 +682,28 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
 // vector load and the increments leave together (one thread walking the ranks
 // waits for a scalar load per rank: 0.8 us for eight).
 __device__ inline void publish_tile(const GemmKArgs& p, int tile_id, int lane) {
-  // the caller's tiles the launch's tile covers: itself, or merge_n in a row
-  int first = tile_id, count = 1, pid_m = 0, pn0 = 0;
-  if (p.merge_n > 1) {
+  // the caller's tiles the launch's tile covers: itself, or a block of merge_m x merge_n (fewer at the edges)
+  const bool merged = p.merge_m * p.merge_n > 1;
+  int first = tile_id, rows = 1, cols = 1, pm0 = 0, pn0 = 0;
+  if (merged) {
     const TileCoord t = tile_map_fast(tile_id, p.num_pid_m, p.num_pid_n, p.G, p.tile_divs);
-    pid_m = t.pid_m;
+    pm0 = t.pid_m * p.merge_m;
     pn0 = t.pid_n * p.merge_n;
-    count = min(p.merge_n, p.flag_num_pid_n - pn0);
+    rows = min(p.merge_m, p.flag_num_pid_m - pm0);
+    cols = min(p.merge_n, p.flag_num_pid_n - pn0);
   }
-  for (int j = 0; j < count; ++j) {
-    if (p.merge_n > 1) first = tile_id_of(pid_m, pn0 + j, p.num_pid_m, p.flag_num_pid_n, p.G);
-    IRIS_GLOBAL int32_t* own = (IRIS_GLOBAL int32_t*)(p.flags + first);
-    for (int r = lane; r < p.ws; r += 64) {
-      if (p.flag_mode == 2 && r == p.cur_rank) continue;
-      IRIS_GLOBAL int32_t* f = own;
-      if (r != p.cur_rank && p.heap_bases != nullptr)
-        f = translate(p.flags + first, p.heap_bases[p.cur_rank], p.heap_bases[r]);
-      flag_add_relaxed(f, 1, p.sys != 0);
+  for (int i = 0; i < rows; ++i)
+    for (int j = 0; j < cols; ++j) {
+      if (merged) first = tile_id_of(pm0 + i, pn0 + j, p.flag_num_pid_m, p.flag_num_pid_n, p.G);
+      IRIS_GLOBAL int32_t* own = (IRIS_GLOBAL int32_t*)(p.flags + first);
+      for (int r = lane; r < p.ws; r += 64) {
+        if (p.flag_mode == 2 && r == p.cur_rank) continue;
+        IRIS_GLOBAL int32_t* f = own;
+        if (r != p.cur_rank && p.heap_bases != nullptr)
+          f = translate(p.flags + first, p.heap_bases[p.cur_rank], p.heap_bases[r]);
+        flag_add_relaxed(f, 1, p.sys != 0);
+      }
     }
-  }
 }
 
 // Split-K hand-over of a partial tile.  The partial keeps the accumulators'

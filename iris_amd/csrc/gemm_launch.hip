@@ -213,42 +213,53 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
 // is no GEMM work to do.
 hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan);
 
-// The plan of a launch.  A caller's tile that is 256 rows tall and narrow (the reference scripts' 256 x 64)
-// makes a large GEMM wait for its operands: every K-step fetches 256 rows of A for 64 columns' worth of work.
-// Where there are enough of them, the launch computes two or four of the caller's tiles, side by side, as one
+// The plan of a launch.  A caller's tile that is narrow or short (the reference scripts' 256 x 64; 128 x 128)
+// makes a large GEMM wait for its operands: a 256 x 64 tile fetches 256 rows of A every K-step for 64 columns'
+// worth of work.  Where there are enough of them, the launch computes a block of the caller's tiles as one
 // 256 x 128 or 256 x 256 tile and raises each one's flag: tile ids and flags are the caller's, which program
-// computes a tile was never observable ([8192,8192] x [8192,1024] in 256 x 64 tiles: 739-762 -> 902 TFLOP/s
+// computes a tile was never observable ([8192,8192] x [8192,1024] in 256 x 64 tiles: 739-762 -> 928 TFLOP/s
 // over the eight ranks of the reference's 07 benchmark).
 hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
-  int merge = 1;
+  int merge_m = 1, merge_n = 1;
   const bool plain = a.variant == 0 && a.split_k == 0 && !a.mm_begin_timestamp && !a.mm_end_timestamp &&
                      !(a.epilogue == IRIS_EPI_ONE_SHOT && a.phase == IRIS_PHASE_FUSED) &&
-                     a.epilogue != IRIS_EPI_ATOMIC_ADD && a.num_sms > 0 && a.block_m == 256 &&
+                     a.epilogue != IRIS_EPI_ATOMIC_ADD && a.num_sms > 0 && (a.block_m == 128 || a.block_m == 256) &&
                      (a.block_n == 64 || a.block_n == 128) && a.M >= 256;
   if (plain) {
-    const int64_t tiles = (int64_t)((a.M + 255) / 256) * ((a.N + a.block_n - 1) / a.block_n);
-    const int up_to = 256 / a.block_n;  // 4 or 2
-    if (tiles >= (int64_t)up_to * a.num_sms)
-      merge = up_to;
-    else if (up_to == 4 && tiles >= 2 * (int64_t)a.num_sms)
-      merge = 2;
+    const int64_t tiles_m = (a.M + a.block_m - 1) / a.block_m, tiles_n = (a.N + a.block_n - 1) / a.block_n;
+    const int mm = 256 / a.block_m;  // 1 or 2
+    const int64_t rows = (tiles_m + mm - 1) / mm;
+    // 256 x 256 or 256 x 128, whichever finishes first among those that give every program a tile: rounds of
+    // tiles times the tile's time (a 256 x 256 tile does twice the work at 1.25 times the rate, as measured)
+    double best = 0;
+    for (int width = 256; width >= 128; width /= 2) {
+      const int mn = width / a.block_n;
+      const int64_t merged_tiles = rows * ((tiles_n + mn - 1) / mn);
+      if (mm * mn == 1 || merged_tiles < a.num_sms) continue;
+      const double cost = (double)((merged_tiles + a.num_sms - 1) / a.num_sms) * (width == 256 ? 1.6 : 1.0);
+      if (best == 0 || cost < best) best = cost, merge_m = mm, merge_n = mn;
+    }
   }
-  if (merge > 1) {
+  if (merge_m * merge_n > 1) {
     iris_gemm_args b = a;
-    b.block_n = a.block_n * merge;
+    b.block_m = a.block_m * merge_m;
+    b.block_n = a.block_n * merge_n;
     Plan merged;
     const hipError_t err = make_plan_body(b, &merged);
     // (only the persistent kernels, unsplit, publish merged tiles)
     if (err == hipSuccess && merged.entry && !merged.skinny && merged.k.split_k == 1 && !merged.k.stream_k &&
         !merged.in_program) {
       *plan = merged;
-      plan->k.merge_n = merge;
+      plan->k.merge_m = merge_m;
+      plan->k.merge_n = merge_n;
+      plan->k.flag_num_pid_m = (a.M + a.block_m - 1) / a.block_m;
       plan->k.flag_num_pid_n = (a.N + a.block_n - 1) / a.block_n;
       return hipSuccess;
     }
   }
   const hipError_t err = make_plan_body(a, plan);
-  plan->k.merge_n = 1;
+  plan->k.merge_m = plan->k.merge_n = 1;
+  plan->k.flag_num_pid_m = plan->k.num_pid_m;
   plan->k.flag_num_pid_n = plan->k.num_pid_n;
   return err;
 }
@@ -706,9 +717,11 @@ extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t
                 : plan.entry && plan.in_program                 ? "+reduce"
                 : plan.entry && plan.k.num_sms > args->num_sms ? "+two_per_cu"
                                                                 : "",
-                plan.entry && plan.k.merge_n == 2   ? "+two_tiles_each"
-                : plan.entry && plan.k.merge_n == 4 ? "+four_tiles_each"
-                                                    : "");
+                !plan.entry                            ? ""
+                : plan.k.merge_m * plan.k.merge_n == 2 ? "+two_tiles_each"
+                : plan.k.merge_m * plan.k.merge_n == 4 ? "+four_tiles_each"
+                : plan.k.merge_m * plan.k.merge_n == 8 ? "+eight_tiles_each"
+                                                       : "");
   return hipSuccess;
 }
 

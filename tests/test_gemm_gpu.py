@@ -522,30 +522,35 @@ def test_build_with_fetching_waves_is_bit_identical_to_the_plain_build(shmem, ep
     assert torch.equal(got[f4_variant].view(width), got[plain_variant].view(width)), f"{f4_name} vs {plain_name}"
 
 
-@pytest.mark.parametrize("M,N,K,BN,grid,ws,suffix", [
-    (1024, 640, 256, 64, 2, 1, "+four_tiles_each"),    # 4 x 10 tiles: the last merged tile of a row covers two
-    (1024, 640, 256, 64, 16, 2, "+two_tiles_each"),    # 40 tiles on 16 programs: pairs; flags on both ranks
-    (520, 392, 328, 128, 3, 1, "+two_tiles_each"),     # 3 x 4 tiles of 256 x 128, ragged edges
-    (1024, 640, 256, 64, 32, 1, ""),                   # too few tiles for the programs: as the caller cut them
+@pytest.mark.parametrize("M,N,K,BM,BN,grid,ws,suffix", [
+    (1024, 640, 256, 256, 64, 2, 1, "+four_tiles_each"),   # 4 x 10 tiles: the last merged tile of a row covers two
+    (1024, 640, 256, 256, 64, 16, 2, "+two_tiles_each"),   # 40 tiles on 16 programs: pairs; flags on both ranks
+    (520, 392, 328, 256, 128, 3, 1, "+two_tiles_each"),    # 3 x 4 tiles of 256 x 128, ragged edges
+    (1024, 640, 256, 256, 64, 32, 1, ""),                  # too few tiles for the programs: as the caller cut them
+    (640, 392, 200, 128, 128, 3, 2, "+four_tiles_each"),   # 5 x 4 tiles of 128 x 128 in blocks of 2 x 2, last row 1 x 2
+    (640, 392, 200, 128, 128, 8, 1, "+two_tiles_each"),    # ... one above the other
+    (640, 200, 136, 128, 64, 3, 1, "+eight_tiles_each"),   # 5 x 4 tiles of 128 x 64 in blocks of 2 x 4
+    (640, 200, 136, 128, 64, 6, 1, "+four_tiles_each"),
 ])
-def test_narrow_tall_tiles_are_computed_several_at_a_time(shmem, M, N, K, BN, grid, ws, suffix):
-    """A caller's 256 x 64 (or 256 x 128) tiles, where there are enough of them,
-    are computed two or four side by side as one tile; every one of the
-    caller's flags is raised exactly once, on every rank, and nothing else."""
+def test_small_tiles_are_computed_several_at_a_time(shmem, M, N, K, BM, BN, grid, ws, suffix):
+    """A caller's 256 x 64, 256 x 128, 128 x 128 or 128 x 64 tiles, where there
+    are enough of them, are computed a block at a time as one 256 x 128 or
+    256 x 256 tile; every one of the caller's flags is raised exactly once,
+    on every rank, and nothing else."""
     dtype = torch.bfloat16
     A, B = make_ab(M, N * ws, K, dtype)
     shards = O.n_shards(A, B, ws)
     a = to_heap(shmem, A)
     bs = [to_heap(shmem, sb) for _, sb in shards]
     cg = shmem.zeros((M, N * ws), dtype=dtype)
-    total = ops.cdiv(M, 256) * ops.cdiv(N, BN)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
     flags = shmem.zeros((total + 5,), dtype=torch.int32)
     hb = shmem.get_heap_bases() if ws > 1 else None
     for r in range(ws):
         for t in (cg, flags):
             shmem.on_rank(t, r).zero_()
     for r in range(ws):
-        args = (a, bs[r], None, shmem.on_rank(cg, r), shmem.on_rank(flags, r), hb, r, ws, grid, 256, BN, 64, 4,
+        args = (a, bs[r], None, shmem.on_rank(cg, r), shmem.on_rank(flags, r), hb, r, ws, grid, BM, BN, 64, 3,
                 ops.EPI_ALL_SCATTER)
         name = ops.gemm_plan_name(*args)
         assert name.endswith(suffix) and (suffix or "tiles_each" not in name), name
