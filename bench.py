@@ -16,6 +16,7 @@ baseline of the same math on the host cores.
 
 import argparse
 import json
+import math
 import os
 import statistics
 import sys
@@ -66,10 +67,14 @@ def parse():
     ap.add_argument("--decoder-tiles", default="",
                     help="decoder workload: only this tile shape, as BLK_MxBLK_N (default: a sweep, and the "
                          "reference examples' default tile 256x64 beside it)")
-    ap.add_argument("--workload", choices=["headline", "atomic", "decoder"], default="headline",
+    ap.add_argument("--shapes-gpus", default="1,2,4,8", help="shapes workload: the GPU counts the GEMMs are cut over")
+    ap.add_argument("--shapes-algorithms", default="all_scatter,one_shot",
+                    help="shapes workload: all_scatter (N-shards) and / or one_shot (K-shards, the producer)")
+    ap.add_argument("--workload", choices=["headline", "atomic", "decoder", "shapes"], default="headline",
                     help="headline: the 8192x8192x1024 shard GEMM + reduce (the metric's configuration); atomic: eight "
                          "K-shard GEMMs adding into one fp32 C; decoder: 6.7B-decoder-shaped shards for M in "
-                         "{1,16,128,512,2048}.  The last two print their own JSON line.")
+                         "{1,16,128,512,2048}; shapes: one rank's shard GEMM at every point of the reference's shape "
+                         "sweep, beside the vendor library's.  The last three print their own JSON line.")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="headline run: skip the atomic-accumulate and decoder-shard summaries")
     ap.add_argument("--no-context", action="store_true",
@@ -317,6 +322,131 @@ def run_atomic(args, emit=True):
     return result
 
 
+# The reference's shape sweep (examples/benchmark/bench_all_shapes.py:103-187): the six GEMMs of
+# dataset/mini.json (m = 8192), each cut over 1, 2, 4 and 8 GPUs, with the tile and group size that
+# dataset/tiling.json holds for the rank's shard shape: (m, k, n / gpus) for the all-scatter, (m, k / gpus, n) for
+# the reduce algorithms.  (n, k) -> gpus -> ((BLK_M, BLK_N, gsize_m) all-scatter, (...) one-shot), as looked up there.
+SWEEP_SHAPES = {
+    (4096, 12288): {1: ((128, 128, 6), (128, 128, 6)), 2: ((256, 256, 6), (128, 128, 6)),
+                    4: ((128, 256, 6), (256, 256, 2)), 8: ((128, 128, 6), (256, 256, 2))},
+    (4096, 14336): {1: ((128, 128, 6), (128, 128, 6)), 2: ((256, 256, 6), (128, 128, 6)),
+                    4: ((128, 256, 6), (256, 256, 2)), 8: ((128, 128, 6), (256, 256, 2))},
+    (3584, 14336): {1: ((128, 256, 6), (128, 256, 6)), 2: ((128, 128, 2), (128, 256, 6)),
+                    4: ((256, 128, 1), (128, 256, 6)), 8: ((256, 64, 1), (128, 256, 6))},
+    (4608, 36864): {1: ((256, 256, 2), (256, 256, 2)), 2: ((256, 256, 6), (256, 256, 2)),
+                    4: ((256, 128, 1), (256, 256, 2)), 8: ((256, 64, 1), (256, 256, 2))},
+    (8192, 28672): {1: ((128, 256, 6), (128, 256, 6)), 2: ((128, 128, 6), (128, 256, 6)),
+                    4: ((256, 256, 6), (128, 256, 6)), 8: ((128, 256, 6), (128, 256, 6))},
+    (8192, 30720): {1: ((128, 256, 6), (128, 256, 6)), 2: ((128, 128, 6), (128, 256, 6)),
+                    4: ((256, 256, 6), (128, 256, 6)), 8: ((128, 256, 6), (128, 256, 6))},
+}
+
+
+def sweep_tile(blk_m, blk_n):
+    """The tile the sweep launches for a tile of the table: it runs 128 x 256 and 128 x 128 entries as 256 x 128
+    (bench_all_shapes.py:161-166)."""
+    return (256, 128) if (blk_m, blk_n) in ((128, 256), (128, 128)) else (blk_m, blk_n)
+
+
+def run_shapes(args, emit=True):
+    """One rank's shard GEMM for every point of the reference's shape sweep, at the sweep's tile, beside the vendor
+    library's plain GEMM on the same shard: the all-scatter ([8192, k] x [k, n / gpus], the tile stored into
+    every rank's C behind its flag) and the producer of the one-shot all-reduce ([8192, k / gpus] x [k / gpus, n]
+    on K-shard views of the whole operands, an fp32 partial behind flags on the other ranks)."""
+    import torch
+
+    import iris_amd
+    from iris_amd import ops
+
+    m = 8192
+    gpus_list = [int(v) for v in args.shapes_gpus.split(",")]
+    points = []
+    for ws in gpus_list:
+        # per rank: A and B of the largest shape (0.6 + 0.5 GB), bf16 C, fp32 partial, flags
+        shmem = iris_amd.iris(2 << 30, virtual_ranks=ws)
+        hb = shmem.get_heap_bases()
+        xcds = ops.default_num_xcds(shmem.get_cu_count(), 256)
+        rank = ws - 1
+        for (n, k), by_gpus in SWEEP_SHAPES.items():
+            if ws not in by_gpus:
+                continue
+            off = shmem.heap_offset
+            a = shmem.zeros((m, k), dtype=torch.bfloat16)
+            bt = shmem.zeros((n, k), dtype=torch.bfloat16)  # B = bt.T: K-contiguous, as the scripts pass it
+            a.normal_(0, 0.02)
+            bt.normal_(0, 0.02)
+            cg = shmem.zeros((m, n), dtype=torch.bfloat16)
+            part = shmem.zeros((m, n), dtype=torch.float32)
+            ns, ks = n // ws, k // ws
+            for algorithm, (bm0, bn0, gsize_m) in zip(("all_scatter", "one_shot"), by_gpus[ws]):
+                if algorithm not in args.shapes_algorithms.split(","):
+                    continue
+                bm, bn = sweep_tile(bm0, bn0)
+                if algorithm == "all_scatter":
+                    a_r, b_r, n_r = a, bt[rank * ns:(rank + 1) * ns].T, ns
+                else:
+                    a_r, b_r, n_r = a[:, rank * ks:(rank + 1) * ks], bt[:, rank * ks:(rank + 1) * ks].T, n
+                flags = shmem.zeros((ops.cdiv(m, bm) * ops.cdiv(n_r, bn),), dtype=torch.int32)
+                # the wrappers' P / locks buffers (benchmark.py:136-142): with them the launcher may split K
+                P = shmem.zeros((256, bm * bn), dtype=torch.float32)
+                locks = shmem.zeros((256,), dtype=torch.int32)
+                if algorithm == "all_scatter":
+                    largs = (a_r, b_r, None, shmem.on_rank(cg, rank), shmem.on_rank(flags, rank), hb, rank, ws, 256,
+                             bm, bn, 64, gsize_m, ops.EPI_ALL_SCATTER)
+                    kw = dict(num_xcds=xcds, partials=P, locks=locks)
+                    got = lambda: shmem.on_rank(cg, 0)[:, rank * ns:(rank + 1) * ns]
+                else:
+                    largs = (a_r, b_r, shmem.on_rank(part, rank), shmem.on_rank(cg, rank),
+                             shmem.on_rank(flags, rank), hb, rank, ws, 256, bm, bn, 64, gsize_m, ops.EPI_ONE_SHOT)
+                    kw = dict(num_xcds=xcds, phase=ops.PHASE_PRODUCE, partials=P, locks=locks)
+                    got = lambda: shmem.on_rank(part, rank)
+                lib = torch.empty((m, n_r), dtype=torch.bfloat16, device="cuda")
+
+                def ours():
+                    ops.gemm_launch(*largs, **kw)
+
+                def library():
+                    torch.matmul(a_r, b_r, out=lib)
+
+                ours()
+                library()
+                torch.cuda.synchronize()
+                # the library's result is bf16 and sums in another order: agreement to two bf16 roundings
+                diff = (got().float() - lib.float()).abs().max().item()
+                scale = lib.float().abs().max().item()
+                assert diff <= 2e-2 * scale, f"{algorithm} n={n} k={k} gpus={ws}: differs from the library's by {diff}"
+                tiles_done = int((shmem.on_rank(flags, 0) > 0).sum().item())
+                assert tiles_done == (flags.numel() if ws > 1 or algorithm == "all_scatter" else 0)
+                flops = 2.0 * m * n_r * a_r.shape[1]
+                t = {}
+                for name, fn in (("ours", ours), ("library", library)):
+                    est = steady_ms(fn, settle_s=0.05, n=3)
+                    t[name] = steady_ms(fn, settle_s=0.1, n=max(5, min(200, int(150.0 / est))))
+                points.append({
+                    "n": n, "k": k, "gpus": ws, "algorithm": algorithm, "shard": [m, n_r, a_r.shape[1]],
+                    "tile": [bm, bn], "gsize_m": gsize_m, "kernel": ops.gemm_plan_name(*largs, **kw),
+                    "split_k": ops.gemm_split_k(*largs, **kw),
+                    "us": round(t["ours"] * 1e3, 1), "tflops": round(flops / t["ours"] / 1e9, 1),
+                    "library_us": round(t["library"] * 1e3, 1), "library_tflops": round(flops / t["library"] / 1e9, 1),
+                    "vs_library": round(t["library"] / t["ours"], 3)})
+                del lib
+            shmem.heap_offset = off
+        del shmem
+    ratios = sorted(p["vs_library"] for p in points)
+    out = {
+        "metric": "shard GEMM + tile-publishing epilogue over the reference's shape sweep: rate against the vendor "
+                  "library's plain GEMM on the same shard (geometric mean)",
+        "value": round(math.exp(sum(math.log(r) for r in ratios) / len(ratios)), 3), "unit": "x",
+        "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "dataset/mini.json's six GEMMs (m = 8192) cut over " + args.shapes_gpus + " GPUs at the "
+                               "tiles of dataset/tiling.json, one rank's share on one GPU with the other ranks' "
+                               "heaps in the same HBM"},
+        "worst": ratios[0], "best": ratios[-1], "points": points}
+    if emit:
+        print(json.dumps(out))
+    return out
+
+
 def run_decoder(args, emit=True):
     """BASELINE config 5: 6.7B-decoder-shaped shards (hidden 4096, FFN 11008,
     1/8 shard = 1376).  Gate/up: [M,4096] x [4096,1376] scattered into every
@@ -515,6 +645,8 @@ def main():
         return run_atomic(args)
     if args.workload == "decoder":
         return run_decoder(args)
+    if args.workload == "shapes":
+        return run_shapes(args)
 
     ws = 8
     # per-rank heap: full-K operands 2 x 128 MiB, bf16 results 2 x 128 MiB, fp32 partial 256 MiB, flags

@@ -121,12 +121,26 @@ struct Mfma<IRIS_DTYPE_BF16> {
   __device__ static inline f32x4 run(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
+  // the same with the accumulator pinned to the accumulation registers (tiles of 256 accumulators a lane:
+  // they fill that half of the register file exactly, and the fragments keep the other half)
+  __device__ static inline void run_acc(vec8 a, vec8 b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  __device__ static inline void first_acc(vec8 a, vec8 b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+  }
 };
 template <>
 struct Mfma<IRIS_DTYPE_F16> {
   using vec8 = f16x8;
   __device__ static inline f32x4 run(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline void run_acc(vec8 a, vec8 b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  __device__ static inline void first_acc(vec8 a, vec8 b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
   }
 };
 
@@ -163,7 +177,7 @@ struct GemmCfg {
   static constexpr bool SPLITK = DMA_ && KSUB % 2 == 0;
   static constexpr bool SPLIT_OWNER = SPLITK && IM * IN * 4 <= 64;
   // Waves per SIMD the register budget is sized for: 256 registers a wave.
-  static constexpr int WPE = 2;
+  static constexpr int WPE = IM * IN * 4 > 128 ? 1 : 2;
   // wave-private epilogue scratch: 32 rows x TN 16-bit elements
   static constexpr int WS_PITCH = TN * 2;
   static constexpr int WS_BYTES = 32 * WS_PITCH;
@@ -179,7 +193,8 @@ struct GemmCfg {
   static_assert(S >= 1, "ring depth");
   static_assert(!DMA || S >= 2, "the DMA ring needs a stage being read and one in flight");
   static_assert(L * (S - 1) <= 63, "vmcnt immediate");
-  static_assert(IM * IN * 4 <= 128, "accumulators of a wave tile: at most 128 registers");
+  static_assert(IM * IN * 4 <= 256, "accumulators of a wave tile: at most 256 registers");
+  static_assert(IM * IN * 4 <= 128 || NW + LW <= 4, "256 accumulators a lane: one wave per SIMD");
   static_assert(TN == 32 || TN == 64 || TN == 128, "wave tile width");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
@@ -462,7 +477,12 @@ template <class Cfg, bool FIRST>
 __device__ inline void mma_row(f32x4 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& f, int cb, int i) {
 #pragma unroll
   for (int j = 0; j < Cfg::IN; ++j) {
-    if constexpr (FIRST) {
+    if constexpr (Cfg::IM * Cfg::IN * 4 > 128) {
+      if constexpr (FIRST)
+        Mfma<Cfg::DT>::first_acc(f.b[cb][j], f.a[i], acc[i][j]);
+      else
+        Mfma<Cfg::DT>::run_acc(f.b[cb][j], f.a[i], acc[i][j]);
+    } else if constexpr (FIRST) {
       const f32x4 z = {0, 0, 0, 0};
       acc[i][j] = Mfma<Cfg::DT>::run(f.b[cb][j], f.a[i], z);
     } else {
@@ -1009,6 +1029,117 @@ __device__ inline void fused_reduce_tile(const GemmKArgs& p, const Item& it, int
 // The kernel
 // ---------------------------------------------------------------------------
 
+// The K loop of the tiles whose wave holds 256 accumulators a lane (256 x 256 as 2 x 2 waves of 128 x 128): one
+// wave per SIMD with the whole register file, the accumulators in its accumulation half.  A 128 x 128 wave tile
+// reads 16 fragments from LDS for 64 MFMAs where the 128 x 64 one reads 12 for 32, and with that the K loop is
+// bound by the matrix cores instead of by LDS.  Stages are 32 deep in a ring of four: step g multiplies the
+// fragments it fetched during step g-1, fetches those of step g+1 from the stage that landed last, and refills
+// the stage it just left with step g+4, one load per block of MFMAs.  Unsplit, one compute tile per logical
+// tile; the flag of a tile is published once the tile's stores have completed.
+//
+// A tuning variant, not the launcher's choice: with one wave per SIMD every load the wave issues holds its
+// MFMAs up, and no fetching wave fits beside a wave of 512 registers.  [8192,7168] x [7168,8192] on zeros:
+// 1.97 PFLOP/s with the loads taken out, 1.79 with every second one, 1.42 with all of them (the eight-wave
+// 256 x 256 tile: 1.53; the vendor library: 2.25); on N(0, 0.02) data 1.29 against 1.36 and 1.63.  The
+// accumulators are pinned to the accumulation registers (Mfma::run_acc): left to the compiler, fragments of
+// the K loop are spilled around them and every reload waits for all loads in flight.
+template <class Cfg, int OP, int ODT>
+__device__ __attribute__((always_inline)) inline void big_tile_main(const GemmKArgs& p, IRIS_LDS char* lds) {
+  static_assert(Cfg::DMA && Cfg::LW == 0 && Cfg::KSUB == 1 && Cfg::S == 4 && Cfg::IM == Cfg::IN, "big-tile K loop");
+  constexpr int L = Cfg::L;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  int pid;
+  if (p.xcd_per > 0) {
+    const int x = blockIdx.x % p.num_xcds, j = blockIdx.x / p.num_xcds;
+    pid = j < p.xcd_per ? x * p.xcd_per + j : p.num_sms * 2;
+  } else {
+    pid = xcd_remap(blockIdx.x, p.num_sms, p.num_xcds);
+  }
+  const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
+  const int n_mine = pid < p.total_tiles ? (p.total_tiles - pid + p.num_sms - 1) / p.num_sms : 0;
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  IRIS_LDS char* ws = lds + Cfg::S * Cfg::STAGE + wave * Cfg::WS_BYTES;
+  const int lrow = lane & 15, lq = lane >> 4;
+  const int xoff = (lq ^ ((lrow / Cfg::RP) % Cfg::CPR)) * 16;
+  const int a_off = (wm * Cfg::TM + lrow) * Cfg::BK * 2 + xoff;
+  const int b_off = Cfg::A_BYTES + (wn * Cfg::TN + lrow) * Cfg::BK * 2 + xoff;
+  const StreamRun sr{0, 0, 0};
+  Loader<Cfg> ld;
+  Frags<Cfg> fr;
+  f32x4 acc[Cfg::IM][Cfg::IN];
+
+  for (int t = 0; t < n_mine; ++t) {
+    const Item it = decode_item<Cfg, false>(p, sr, pid, t);
+    if (p.ts_begin && tid == 0)
+      __hip_atomic_fetch_min((IRIS_GLOBAL unsigned long long*)(p.ts_begin + it.tile_id),
+                             (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 0; i < Cfg::IM; ++i)
+#pragma unroll
+      for (int j = 0; j < Cfg::IN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (nk > 0) {
+      // steps 0..3 into the four stages (steps past K fetch nothing)
+      ld.setup(p, it, wave, lane, 0);
+      ld.issue(p, lds, 0, wave);
+#pragma unroll
+      for (int s = 1; s < Cfg::S; ++s) {
+        ld.before_step(s, wave, lane);
+        ld.issue(p, lds + s * Cfg::STAGE, s, wave);
+      }
+      IRIS_WAIT_VMCNT(L * (Cfg::S - 1));
+      block_barrier_raw();
+      load_all<Cfg>(lds + a_off, lds + b_off, fr, 0);
+
+      auto step = [&](int g, auto par_tag) __attribute__((always_inline)) {
+        constexpr int cb = decltype(par_tag)::value;
+        mma_row<Cfg, false>(acc, fr, cb, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        // this wave's part of stage g+1 has landed (steps g+2 and g+3 may be in flight), and its reads of
+        // stage g, the fragments it is multiplying, have returned
+        IRIS_WAIT_VMCNT(L * (Cfg::S - 2));
+        IRIS_WAIT_LGKMCNT0();
+        block_barrier_raw();
+        const IRIS_LDS char* nst = lds + ((g + 1) & (Cfg::S - 1)) * Cfg::STAGE;
+        IRIS_LDS char* rst = lds + (g & (Cfg::S - 1)) * Cfg::STAGE;
+        ld.before_step(g + Cfg::S, wave, lane);
+        fr.a[0] = load_a<Cfg>(nst + a_off, 0);
+        fr.b[cb ^ 1][0] = load_b<Cfg>(nst + b_off, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 1; i < Cfg::IM; ++i) {
+          mma_row<Cfg, false>(acc, fr, cb, i);
+          fr.a[i] = load_a<Cfg>(nst + a_off, i);
+          fr.b[cb ^ 1][i] = load_b<Cfg>(nst + b_off, i);
+          // every wave is past its reads of stage g: refill it with step g+4, the loads shared out over the blocks
+#pragma unroll
+          for (int q = (i - 1) * L / (Cfg::IM - 1); q < i * L / (Cfg::IM - 1); ++q)
+            ld.issue_at(p, rst, g + Cfg::S, wave, q);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      };
+      int g = 0;
+      for (; g + 1 < nk; g += 2) {
+        step(g, std::integral_constant<int, 0>{});
+        step(g + 1, std::integral_constant<int, 1>{});
+      }
+      if (g < nk) step(g, std::integral_constant<int, 0>{});
+      // the last MFMAs' results must have left the matrix cores before they are read
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    }
+    store_acc<Cfg, OP, ODT>(p, acc, ws, it.m0 + wm * Cfg::TM, it.n0 + wn * Cfg::TN, it.m_end, it.n_end, lane);
+    // this wave's stores have completed, none of its loads is still writing a stage, and it has read all it will
+    IRIS_WAIT_VMCNT(0);
+    IRIS_WAIT_LGKMCNT0();
+    __syncthreads();
+    if (p.flag_mode != 0 && wave == 0) publish_tile(p, it.tile_id, lane);
+    if (p.ts_end && tid == 0)
+      __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + it.tile_id),
+                             (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 // SPLIT: the split-K build of the kernel (only launched with p.split_k > 1);
 // the plain build carries none of its code or state.
 // FUSED: the one-shot epilogue as the reference program runs it
@@ -1020,6 +1151,11 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(Cf
 gemm_persistent_kernel(const GemmKArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   IRIS_LDS char* lds = (IRIS_LDS char*)lds_raw;
+  if constexpr (Cfg::IM * Cfg::IN * 4 > 128) {
+    static_assert(!SPLIT, "the 256-accumulator tiles have no split-K build");
+    if constexpr (!FUSED) big_tile_main<Cfg, OP, ODT>(p, lds);  // (no build with the reduce inside either)
+    return;
+  }
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -178,7 +178,10 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
       // the K-steps a quarter shorter and left the hand-over as it was: on the same shapes
       // stream-K now ties with split-K (66 tiles: 27.9 against 27.6 us in three parts) or
       // loses (88 tiles: 33.2 against 31.9 in two parts; 132 tiles: 41.0 against 37.6 unsplit;
-      // more tiles than programs: 80 against 54).
+      // more tiles than programs: 80 against 54).  Nor does it pay where the walk is long and the last round
+      // of tiles leaves most programs idle ([8192,36864] x [36864,576] in 288 tiles of 256 x 64 on 256
+      // programs: 940 against 805 us): programs that start at different depths of K no longer fetch the
+      // panels their neighbours fetch at the same time, and the operands come from HBM several times over.
     }
   } else if (a.split_k > 1 || a.split_k == IRIS_GEMM_SPLIT_STREAM_K) {
     return hipErrorInvalidValue;  // forced, but no workspace
@@ -469,7 +472,13 @@ hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan) {
   // A split launch of a 128-accumulator tile: the fetch state of the `_f4` build spills next
   // to the hand-over's registers ([128,4096] x [4096,1376] as one 256 x 128 tile row in 16
   // parts: 24.0 us against the plain tile's 21.2).
-  if (k.split_k != 1 && twin && !pick->split_owner && twin->bk == pick->bk) plan->entry = twin;
+  // (With 32 K-steps or more a part the spills are paid once and the K loop decides: [8192,12288] x
+  // [12288,512] as 128 tiles of 256 x 128 in two parts.)
+  {
+    const int nk = (a.K + pick->bk - 1) / pick->bk;
+    if (k.split_k != 1 && twin && !pick->split_owner && twin->bk == pick->bk && nk / k.split_k < 32)
+      plan->entry = twin;
+  }
   return hipSuccess;
 }
 

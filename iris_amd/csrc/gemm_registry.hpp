@@ -38,7 +38,7 @@ template <class Cfg, int OP, int ODT>
 constexpr GemmKernelFn fused_fn() {
   // (the tiles with fetching waves have no such build: the reduce wants the registers their
   // fetch state takes, and the launcher takes the plain tile of the same shape instead)
-  if constexpr ((OP == OP_STORE16 || OP == OP_STORE32) && Cfg::LW == 0)
+  if constexpr ((OP == OP_STORE16 || OP == OP_STORE32) && Cfg::LW == 0 && Cfg::IM * Cfg::IN * 4 <= 128)
     return &gemm_persistent_kernel<Cfg, OP, ODT, false, true>;
   else
     return nullptr;
@@ -93,7 +93,8 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   X(DT, OP, 128, 256, 64, 2, 4, 2, true, 0, 1, "128x256x64_w2x4_s2")         \
   X(DT, OP, 128, 128, 32, 2, 2, 4, true, 0, 0, "128x128x32_w2x2_s4")         \
   X(DT, OP, 64, 64, 64, 2, 2, 4, true, 4, 1, "64x64x64_w2x2_s4_f4")          \
-  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")
+  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")        \
+  X(DT, OP, 256, 256, 32, 2, 2, 4, true, 0, 0, "256x256x32_w2x2_s4")
 
 #define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, SPLIT, NAME) \
   make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP>(NAME),
