@@ -845,10 +845,17 @@ def main():
                 "split_k_down", "down_us", "down_tflops", "reduce_us", "reduce_GBps", "gate_up_one_destination_us",
                 "gate_up_without_fetching_waves_us",
                 "library_gate_up_us", "library_down_us", "at_reference_default_tile_256x64")
+        args.shapes_gpus = "8"  # (the whole sweep, 1 to 8 GPUs, is the --workload shapes run)
+        sweep = run_shapes(args, emit=False)
         result["other_workloads"] = {
             "atomic_accumulate": {k: at[k] for k in ("value", "unit", "ms_per_step", "atomic_updates_per_s",
                                                      "atomic_ceiling", "config")},
             "decoder_shards": {"config": dec["config"], "per_M": [{k: r[k] for k in keep} for r in dec["per_M"]]},
+            "shape_sweep_8_gpus": {"vs_library_geomean": sweep["value"], "worst": sweep["worst"],
+                                   "best": sweep["best"], "config": sweep["config"],
+                                   "points": [{k: pt[k] for k in ("algorithm", "shard", "tile", "kernel", "split_k",
+                                                                  "us", "tflops", "library_us", "vs_library")}
+                                              for pt in sweep["points"]]},
         }
 
     if not args.no_cpu:
