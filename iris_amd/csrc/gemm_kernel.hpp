@@ -64,6 +64,9 @@ struct GemmKArgs {
   // (neighbouring tiles, whose operand panels its L2 then fetches once).
   int xcd_per;
   int num_pid_m, num_pid_n, total_tiles;
+  // The launch covers tiles tile_base .. tile_base + total_tiles - 1 of the num_pid_m x num_pid_n grid (a launch
+  // over all of them has base 0; a GEMM whose last round of tiles is split over the idle programs is two).
+  int tile_base;
   int sub_m, sub_n;  // compute tiles per logical tile
   // the launch's divisors, for the tile decode (see FastDiv)
   TileDivs tile_divs;
@@ -276,7 +279,7 @@ __device__ inline Item decode_item(const GemmKArgs& p, const StreamRun& sr, int 
   if constexpr (SPLIT) {
     // one compute tile per logical tile; the program's run touches tiles
     // tile0, tile0 + 1, ...
-    it.tile_id = sr.tile0 + item;
+    it.tile_id = p.tile_base + sr.tile0 + item;
     const TileCoord tc = tile_map_fast(it.tile_id, p.num_pid_m, p.num_pid_n, p.G, p.tile_divs);
     it.lm0 = it.m0 = tc.pid_m * p.BM;
     it.ln0 = it.n0 = tc.pid_n * p.BN;
@@ -287,7 +290,7 @@ __device__ inline Item decode_item(const GemmKArgs& p, const StreamRun& sr, int 
   }
   const int ti = (int)fast_div((uint32_t)item, p.div_subs);
   const int s = item - ti * subs;
-  it.tile_id = pid + ti * p.num_sms;
+  it.tile_id = p.tile_base + pid + ti * p.num_sms;
   const TileCoord tc = tile_map_fast(it.tile_id, p.num_pid_m, p.num_pid_n, p.G, p.tile_divs);
   it.lm0 = tc.pid_m * p.BM;
   it.ln0 = tc.pid_n * p.BN;

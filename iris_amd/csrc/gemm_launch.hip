@@ -1,5 +1,6 @@
 // C-ABI launcher of the persistent shard GEMM (include/iris_amd.h).
 #include <cstdio>
+#include <cstring>
 #include <cstdlib>
 #include <mutex>
 #include <utility>
@@ -58,6 +59,10 @@ struct Plan {
   GemmKernelFn skinny = nullptr;
   int skinny_grid = 0, skinny_grid_y = 1, skinny_lds = 0;
   int skinny_rb = 1, skinny_cb = 1;  // blocks of 16 rows / 16 columns a workgroup of the few-rows kernel takes
+  // a second launch of the entry's split-K build behind the first: the tiles of the last round, K shared out
+  // over the programs that round would leave idle
+  int last_round = 0;
+  GemmKArgs k_last{};
 };
 
 int dbg() {
@@ -211,10 +216,64 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
   return hipSuccess;
 }
 
+// The launch's divisors as multiply-high constants, and how its items are dealt to the XCDs.
+void launch_constants(const iris_gemm_args& a, const GemmKernelEntry& pick, GemmKArgs* kp) {
+  GemmKArgs& k = *kp;
+  const int nk = (a.K + pick.bk - 1) / pick.bk;
+  const uint64_t items = (uint64_t)k.total_tiles * k.sub_m * k.sub_n + 1;
+  k.tile_divs = make_tile_divs(k.num_pid_m, k.num_pid_n, k.G);
+  k.div_subs = make_fast_div((uint32_t)(k.sub_m * k.sub_n), items);
+  k.div_sub_n = make_fast_div((uint32_t)k.sub_n, items);
+  k.div_split = make_fast_div((uint32_t)k.split_k, (uint64_t)a.num_sms + 1);
+  k.div_nk = make_fast_div((uint32_t)(nk > 0 ? nk : 1), (uint64_t)k.total_tiles * (nk > 0 ? nk : 1) + 1);
+  // Fewer (tile, part) items than programs: deal them to the XCDs evenly, in
+  // consecutive runs, instead of filling the first XCDs and idling the rest.
+  // (under stream-K every program has a run: the reference's XCD remap stays)
+  const int64_t work = (int64_t)k.total_tiles * k.split_k;
+  k.xcd_per = 0;
+  if (!k.stream_k && a.num_xcds > 1 && work < a.num_sms) k.xcd_per = (int)((work + a.num_xcds - 1) / a.num_xcds);
+}
+
 // Validate `a` and build the launch plan.  Returns hipSuccess,
 // hipErrorInvalidValue, or a pseudo-success with entry == nullptr when there
 // is no GEMM work to do.
 hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan);
+
+// A long GEMM whose tiles are a few more than a multiple of the programs spends a whole round on those few:
+// 288 tiles on 256 programs take two rounds for 1.125 rounds of work.  Where a tile's walk over K is long
+// and the caller brought the split-K workspace, the plan becomes two launches on the stream: the full rounds
+// as they are, then the tiles of the last round with K shared out over the programs it would leave idle
+// (every part at the same depths of K as its neighbours', so the operand panels are still fetched together;
+// stream-K, which would even out the rounds too, loses that and is slower here).
+void split_last_round(const iris_gemm_args& a, Plan* plan) {
+  GemmKArgs& k = plan->k;
+  const GemmKernelEntry* e = plan->entry;
+  plan->last_round = 0;
+  if (!e || plan->skinny || plan->in_program || k.split_k != 1 || k.stream_k || k.sub_m != 1 || k.sub_n != 1) return;
+  if (a.split_k != 0 || a.variant != 0 || a.mm_begin_timestamp || a.mm_end_timestamp) return;
+  if (!a.partials || !a.locks || !e->splitk || !e->fn_split || k.num_sms != a.num_sms) return;
+  if (a.num_sms > current_cu_count() || a.partials_slot_elems < (int64_t)e->cm * e->cn) return;
+  const int programs = a.num_sms, rounds = k.total_tiles / programs, last = k.total_tiles - rounds * programs;
+  if (rounds < 1 || last == 0 || last * 2 > programs) return;
+  const int nk = (a.K + e->bk - 1) / e->bk;
+  // parts of at least 32 K-steps: the build with fetching waves of a split 128-accumulator tile needs them
+  // to pay for its spills, and the second launch's start must be little beside a part's walk
+  int parts = programs / last;
+  if (parts > 16) parts = 16;
+  if (parts > nk / 32) parts = nk / 32;
+  if (parts < 2) return;
+  iris_gemm_args forced = a;
+  forced.split_k = parts;
+  GemmKArgs t = k;
+  t.tile_base = rounds * programs;
+  t.total_tiles = last;
+  if (plan_split(forced, *e, false, &t) != hipSuccess || t.split_k != parts) return;
+  launch_constants(forced, *e, &t);
+  k.total_tiles = rounds * programs;
+  launch_constants(a, *e, &k);
+  plan->k_last = t;
+  plan->last_round = 1;
+}
 
 // The plan of a launch.  A caller's tile that is narrow or short (the reference scripts' 256 x 64; 128 x 128)
 // makes a large GEMM wait for its operands: a 256 x 64 tile fetches 256 rows of A every K-step for 64 columns'
@@ -257,6 +316,7 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
       plan->k.merge_n = merge_n;
       plan->k.flag_num_pid_m = (a.M + a.block_m - 1) / a.block_m;
       plan->k.flag_num_pid_n = (a.N + a.block_n - 1) / a.block_n;
+      split_last_round(b, plan);
       return hipSuccess;
     }
   }
@@ -264,6 +324,7 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
   plan->k.merge_m = plan->k.merge_n = 1;
   plan->k.flag_num_pid_m = plan->k.num_pid_m;
   plan->k.flag_num_pid_n = plan->k.num_pid_n;
+  if (err == hipSuccess) split_last_round(a, plan);
   return err;
 }
 
@@ -435,22 +496,9 @@ hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan) {
   plan->entry = pick;
 
   const hipError_t err = plan_split(a, *pick, plan->in_program != 0, &k);
-  {
-    // the launch's divisors as multiply-high constants
-    const int nk = (a.K + pick->bk - 1) / pick->bk;
-    const uint64_t items = (uint64_t)k.total_tiles * k.sub_m * k.sub_n + 1;
-    k.tile_divs = make_tile_divs(k.num_pid_m, k.num_pid_n, k.G);
-    k.div_subs = make_fast_div((uint32_t)(k.sub_m * k.sub_n), items);
-    k.div_sub_n = make_fast_div((uint32_t)k.sub_n, items);
-    k.div_split = make_fast_div((uint32_t)k.split_k, (uint64_t)a.num_sms + 1);
-    k.div_nk = make_fast_div((uint32_t)(nk > 0 ? nk : 1), (uint64_t)k.total_tiles * (nk > 0 ? nk : 1) + 1);
-  }
+  launch_constants(a, *pick, &k);
   // (under stream-K every program has a run: the reference's XCD remap stays)
   if (err != hipSuccess || k.stream_k) return err;
-  // Fewer (tile, part) items than programs: deal them to the XCDs evenly, in
-  // consecutive runs, instead of filling the first XCDs and idling the rest.
-  const int64_t work = (int64_t)k.total_tiles * k.split_k;
-  if (a.num_xcds > 1 && work < a.num_sms) k.xcd_per = (int)((work + a.num_xcds - 1) / a.num_xcds);
   // A tile whose stages take at most half a CU's LDS runs one wave per SIMD
   // and has every instruction of a K-step on its critical path.  A launch
   // that owns the whole device (one program per CU or more) and has at least
@@ -570,6 +618,18 @@ hipError_t run_plan(const Plan& plan, const iris_gemm_args& args, void* stream) 
     hipLaunchKernelGGL(fn, dim3(plan.k.num_sms), dim3(e->threads), e->lds_bytes, s, plan.k);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
+    if (plan.last_round) {
+      if (e->lds_bytes > 64 * 1024) {
+        err = ensure_lds(e->fn_split, e->lds_bytes);
+        if (err != hipSuccess) return err;
+      }
+      if (dbg())
+        std::fprintf(stderr, "[iris_amd] gemm %s: last round, tiles %d..%d in %d parts\n", e->name,
+                     plan.k_last.tile_base, plan.k_last.tile_base + plan.k_last.total_tiles - 1, plan.k_last.split_k);
+      hipLaunchKernelGGL(e->fn_split, dim3(plan.k_last.num_sms), dim3(e->threads), e->lds_bytes, s, plan.k_last);
+      err = hipGetLastError();
+      if (err != hipSuccess) return err;
+    }
   }
   if (plan.fused_reduce) {
     // The consumer half of the one-shot epilogue runs as a second kernel on
@@ -731,6 +791,10 @@ extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t
                 : plan.k.merge_m * plan.k.merge_n == 4 ? "+four_tiles_each"
                 : plan.k.merge_m * plan.k.merge_n == 8 ? "+eight_tiles_each"
                                                        : "");
+  if (plan.last_round) {
+    const size_t n = std::strlen(buf);
+    std::snprintf(buf + n, len > n ? len - n : 0, "+last_round_in_%d_parts", plan.k_last.split_k);
+  }
   return hipSuccess;
 }
 

@@ -709,6 +709,46 @@ def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
         assert flags2.cpu().tolist()[:4] == [1] * 4 and int(locks.abs().max().item()) == 0
 
 
+@pytest.mark.parametrize("M,N,BN,ws,suffix", [
+    # 18 tiles on 16 programs: 16 whole, 2 in four parts (the owner's hand-over)
+    (512, 576, 64, 1, "256x64x64_w4x1_s3_f4+last_round_in_4_parts"),
+    # 18 tiles: 16 whole, 2 in four parts (the sliced hand-over), on two ranks
+    (512, 1152, 128, 2, "256x128x64_w2x2_s3_f4+last_round_in_4_parts"),
+])
+def test_a_short_last_round_of_long_tiles_is_split_over_the_idle_programs(shmem, M, N, BN, ws, suffix):
+    """Tiles a few more than a multiple of the programs, K long: the full rounds
+    run as they are and a second launch shares K of the last round's tiles
+    out; values, every flag once on every rank, workspace left clean."""
+    K, grid, dtype = 8192, 16, torch.bfloat16
+    A, B = make_ab(M, N * ws, K, dtype)
+    shards = O.n_shards(A, B, ws)
+    a = to_heap(shmem, A)
+    bs = [to_heap(shmem, sb) for _, sb in shards]
+    cg = shmem.zeros((M, N * ws), dtype=dtype)
+    total = ops.cdiv(M, 256) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total + 3,), dtype=torch.int32)
+    partials, locks = split_workspace(shmem, grid, 256, BN)
+    hb = shmem.get_heap_bases() if ws > 1 else None
+    for r in range(ws):
+        for t in (cg, flags):
+            shmem.on_rank(t, r).zero_()
+    for r in range(ws):
+        args = (a, bs[r], None, shmem.on_rank(cg, r), shmem.on_rank(flags, r), hb, r, ws, grid, 256, BN, 64, 4,
+                ops.EPI_ALL_SCATTER)
+        assert ops.gemm_plan_name(*args, partials=partials, locks=locks) == suffix
+        assert "last_round" not in ops.gemm_plan_name(*args)                    # no workspace: as before
+        ops.gemm_launch(*args, partials=partials, locks=locks)
+        torch.cuda.synchronize()
+        assert int(locks.abs().max().item()) == 0
+    want = O.all_scatter(shards, dtype)
+    for r in range(ws):
+        check_close(shmem.on_rank(cg, r), want, f"rank {r}")
+        assert shmem.on_rank(flags, r).cpu().tolist() == [ws] * total + [0] * 3
+    # a shorter K keeps the one launch
+    assert "last_round" not in ops.gemm_plan_name(a[:, :2048], bs[0][:2048], None, cg, flags, hb, 0, ws, grid, 256, BN, 64,
+                                                  4, ops.EPI_ALL_SCATTER, partials=partials, locks=locks)
+
+
 STREAM_K_CASES = [
     # M, N, K, BLK_M, BLK_N, grid, dtype
     (2048, 1376, 1024, 128, 128, 256, torch.bfloat16),  # 176 tiles x 16 steps on 256 programs: runs of 11
