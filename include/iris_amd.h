@@ -226,7 +226,10 @@ int iris_gemm_split_k(const iris_gemm_args* args, int* split_k);
  * followed by "+stream_k", "+reduce" (the in-program reduce) or "+two_per_cu"
  * (two programs a CU), and by "+two_tiles_each" / "+four_tiles_each" /
  * "+eight_tiles_each" where the launch computes a block of that many of the
- * caller's tiles as one (each tile keeps its own id and flag). */
+ * caller's tiles as one (each tile keeps its own id and flag), and by
+ * "+last_round_in_N_parts" where a second launch shares K of the last round's
+ * tiles out over the programs that round would leave idle (needs partials and
+ * locks). */
 int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t len);
 
 /* Name of tuning variant `variant` (1-based) of the kernel list used for
