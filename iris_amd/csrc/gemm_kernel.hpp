@@ -63,6 +63,11 @@ struct GemmKArgs {
   // whole XCDs idle then; instead each XCD takes xcd_per consecutive items
   // (neighbouring tiles, whose operand panels its L2 then fetches once).
   int xcd_per;
+  // > 0 (split-K launches with long parts; the value is total_tiles): the programs are numbered part by part
+  // rather than tile by tile, so that an XCD's programs walk the same range of K over neighbouring tiles and
+  // its L2 fetches each operand panel of that range once.  (Tile by tile, every program of an XCD walks a
+  // different range and nothing is shared: the operands then come from HBM once per tile.)
+  int part_major;
   int num_pid_m, num_pid_n, total_tiles;
   // The launch covers tiles tile_base .. tile_base + total_tiles - 1 of the num_pid_m x num_pid_n grid (a launch
   // over all of them has base 0; a GEMM whose last round of tiles is split over the idle programs is two).
@@ -1177,6 +1182,12 @@ gemm_persistent_kernel(const GemmKArgs p) {
     pid = j < p.xcd_per ? x * p.xcd_per + j : p.num_sms * 2;  // (past every item: nothing to do)
   } else {
     pid = xcd_remap(blockIdx.x, p.num_sms, p.num_xcds);
+  }
+  if constexpr (SPLIT) {
+    if (p.part_major > 0 && pid < p.part_major * p.split_k) {
+      const int part = pid / p.part_major, tile = pid - part * p.part_major;
+      pid = tile * p.split_k + part;
+    }
   }
 
   constexpr bool split = SPLIT;

@@ -230,6 +230,9 @@ void launch_constants(const iris_gemm_args& a, const GemmKernelEntry& pick, Gemm
   // consecutive runs, instead of filling the first XCDs and idling the rest.
   // (under stream-K every program has a run: the reference's XCD remap stays)
   const int64_t work = (int64_t)k.total_tiles * k.split_k;
+  // parts of 32 K-steps or more: the programs part by part (see GemmKArgs::part_major; the short walks of
+  // the decoder shapes were tuned tile by tile and stay so)
+  k.part_major = (k.split_k > 1 && !k.stream_k && nk / k.split_k >= 32) ? k.total_tiles : 0;
   k.xcd_per = 0;
   if (!k.stream_k && a.num_xcds > 1 && work < a.num_sms) k.xcd_per = (int)((work + a.num_xcds - 1) / a.num_xcds);
 }
