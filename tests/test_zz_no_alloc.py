@@ -45,6 +45,28 @@ def test_noalloc_matches_the_workspace_launch_twice(shmem):
     run_pair(shmem, 128, 128, 512, 64, 64, 4, torch.float16, ops.SPLIT_STREAM_K, ops.SPLIT_STREAM_K)
 
 
+def test_noalloc_last_round_split_matches_the_workspace_launch(shmem):
+    # 18 tiles of 128 x 128 on 16 programs, K = 4096: 16 whole tiles, then the last two in two parts each,
+    # as two launches; the second one's partials and locks live in the library's array
+    dtype, M, N, K, grid = torch.bfloat16, 384, 768, 4096, 16
+    A, B = make_ab(M, N, K, dtype, seed=11)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    partials = shmem.zeros((grid, 128 * 128), dtype=torch.float32)
+    locks = shmem.zeros((grid,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+    args = lambda cg, flags: (a, b, None, cg, flags, hb, 0, 1, grid, 128, 128, 64, 2, ops.EPI_ALL_SCATTER)
+    for _ in range(2):
+        cg_ws, cg_na = shmem.zeros((M, N), dtype=dtype), shmem.zeros((M, N), dtype=dtype)
+        f_ws, f_na = shmem.zeros((18,), dtype=torch.int32), shmem.zeros((18,), dtype=torch.int32)
+        assert ops.gemm_plan_name(*args(cg_ws, f_ws), partials=partials, locks=locks).endswith("+last_round_in_2_parts")
+        ops.gemm_launch(*args(cg_ws, f_ws), partials=partials, locks=locks)
+        ops.gemm_launch(*args(cg_na, f_na), noalloc=True)
+        torch.cuda.synchronize()
+        check_close(cg_ws, O.shard_gemm(A, B, dtype), "workspace launch vs oracle")
+        assert torch.equal(cg_na.cpu().view(torch.int16), cg_ws.cpu().view(torch.int16))
+        assert f_na.cpu().tolist() == f_ws.cpu().tolist() == [1] * 18 and int(locks.abs().max().item()) == 0
+
+
 def test_noalloc_few_rows_counters_and_launcher_choice(shmem):
     # the few-rows kernel counts a tile's arrivals in the same array
     dtype = torch.bfloat16
