@@ -734,7 +734,7 @@ extern "C" int iris_gemm_launch_noalloc(const iris_gemm_args* args, void* stream
   // The array keeps what the last call left: the locks must start at zero (a
   // wait that timed out leaves one raised).  A fill kernel, not a memset, so
   // that the call can be recorded into a HIP graph.
-  const bool uses_locks = (plan.skinny && plan.k.flag_mode != 0) || (plan.entry && (plan.k.split_k > 1 || plan.k.stream_k));
+  const bool uses_locks = (plan.skinny && plan.k.flag_mode != 0) || (plan.entry && (plan.k.split_k > 1 || plan.k.stream_k || plan.last_round));
   if (uses_locks) {
     hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), a.locks, 0,
                        (int)(NOALLOC_LOCK_BYTES / sizeof(int32_t)));
