@@ -69,8 +69,10 @@ struct GemmKArgs {
   // different range and nothing is shared: the operands then come from HBM once per tile.)
   int part_major;
   int num_pid_m, num_pid_n, total_tiles;
-  // The launch covers tiles tile_base .. tile_base + total_tiles - 1 of the num_pid_m x num_pid_n grid (a launch
-  // over all of them has base 0; a GEMM whose last round of tiles is split over the idle programs is two).
+  // The launch covers tiles tile_base .. tile_base + total_tiles - 1 of the num_pid_m x num_pid_n grid.  Only the
+  // split-K builds read it: a GEMM whose last round of tiles is split over the idle programs is an unsplit launch
+  // from tile 0 and a split one from tile_base.  (The unsplit 256 x 256 kernel with one more scalar live across
+  // its K loop ran 1.6 % slower on the headline shape.)
   int tile_base;
   int sub_m, sub_n;  // compute tiles per logical tile
   // the launch's divisors, for the tile decode (see FastDiv)
@@ -295,7 +297,7 @@ __device__ inline Item decode_item(const GemmKArgs& p, const StreamRun& sr, int 
   }
   const int ti = (int)fast_div((uint32_t)item, p.div_subs);
   const int s = item - ti * subs;
-  it.tile_id = p.tile_base + pid + ti * p.num_sms;
+  it.tile_id = pid + ti * p.num_sms;  // (the unsplit builds only run launches whose tile_base is 0)
   const TileCoord tc = tile_map_fast(it.tile_id, p.num_pid_m, p.num_pid_n, p.G, p.tile_divs);
   it.lm0 = tc.pid_m * p.BM;
   it.ln0 = tc.pid_n * p.BN;
