@@ -5,6 +5,7 @@ namespace iris_amd {
 
 IRIS_GEMM_VARIANTS(IRIS_GEMM_INSTANTIATE, IRIS_DTYPE_F16, OP_STORE16)
 IRIS_GEMM_VARIANTS(IRIS_GEMM_INSTANTIATE_FUSED, IRIS_DTYPE_F16, OP_STORE16)
+IRIS_GEMM_INSTANTIATE_MERGED(IRIS_DTYPE_F16, OP_STORE16)
 
 static const GemmKernelEntry k_entries[] = {IRIS_GEMM_VARIANTS(IRIS_GEMM_ENTRY, IRIS_DTYPE_F16, OP_STORE16)};
 

@@ -63,26 +63,12 @@ struct GemmKArgs {
   // whole XCDs idle then; instead each XCD takes xcd_per consecutive items
   // (neighbouring tiles, whose operand panels its L2 then fetches once).
   int xcd_per;
-  // > 0 (split-K launches with long parts; the value is total_tiles): the programs are numbered part by part
-  // rather than tile by tile, so that an XCD's programs walk the same range of K over neighbouring tiles and
-  // its L2 fetches each operand panel of that range once.  (Tile by tile, every program of an XCD walks a
-  // different range and nothing is shared: the operands then come from HBM once per tile.)
-  int part_major;
   int num_pid_m, num_pid_n, total_tiles;
-  // The launch covers tiles tile_base .. tile_base + total_tiles - 1 of the num_pid_m x num_pid_n grid.  Only the
-  // split-K builds read it: a GEMM whose last round of tiles is split over the idle programs is an unsplit launch
-  // from tile 0 and a split one from tile_base.  (The unsplit 256 x 256 kernel with one more scalar live across
-  // its K loop ran 1.6 % slower on the headline shape.)
-  int tile_base;
   int sub_m, sub_n;  // compute tiles per logical tile
   // the launch's divisors, for the tile decode (see FastDiv)
   TileDivs tile_divs;
   FastDiv div_subs, div_sub_n;  // sub_m * sub_n, sub_n
   FastDiv div_split, div_nk;    // split_k; K-steps of a tile (stream-K runs)
-  // merge_m * merge_n > 1: the launch's tiles (BM, BN, num_pid_m, num_pid_n, tile ids above) are merge_m x
-  // merge_n of the caller's tiles; the flags stay the caller's, one per tile of BM / merge_m x BN / merge_n,
-  // numbered over flag_num_pid_m x flag_num_pid_n tiles
-  int merge_m, merge_n, flag_num_pid_m, flag_num_pid_n;
   int dest_all;      // write `out` on every rank's heap (else on this rank only)
   int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
   int sys;           // flag atomics at system scope (else agent)
@@ -121,6 +107,23 @@ struct GemmKArgs {
   int64_t sgm, sgn;  // strides of `cg`, elements
   int cg_dt;         // element type of `cg`
   int fused_vec;     // 16-byte strips allowed on `out` and `cg` in the in-program reduce
+
+  // What only some builds read comes last, so that the others find every field where it was (the unsplit
+  // 256 x 256 kernel is sensitive to the scalars it keeps across its K loop).
+  // > 0 (split-K launches with long parts; the value is total_tiles): the programs are numbered part by part
+  // rather than tile by tile, so that an XCD's programs walk the same range of K over neighbouring tiles and
+  // its L2 fetches each operand panel of that range once.  (Tile by tile, every program of an XCD walks a
+  // different range and nothing is shared: the operands then come from HBM once per tile.)
+  int part_major;
+  // The launch covers tiles tile_base .. tile_base + total_tiles - 1 of the num_pid_m x num_pid_n grid.  Only the
+  // split-K builds read it: a GEMM whose last round of tiles is split over the idle programs is an unsplit launch
+  // from tile 0 and a split one from tile_base.  (The unsplit 256 x 256 kernel with one more scalar live across
+  // its K loop ran 1.6 % slower on the headline shape.)
+  int tile_base;
+  // merge_m * merge_n > 1: the launch's tiles (BM, BN, num_pid_m, num_pid_n, tile ids above) are merge_m x
+  // merge_n of the caller's tiles; the flags stay the caller's, one per tile of BM / merge_m x BN / merge_n,
+  // numbered over flag_num_pid_m x flag_num_pid_n tiles
+  int merge_m, merge_n, flag_num_pid_m, flag_num_pid_n;
 };
 
 template <int DT>
@@ -711,11 +714,14 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
 // Lane l takes ranks l, l + 64, ...: the ranks' heap bases come in with one
 // vector load and the increments leave together (one thread walking the ranks
 // waits for a scalar load per rank: 0.8 us for eight).
+template <bool MERGED = false>
 __device__ inline void publish_tile(const GemmKArgs& p, int tile_id, int lane) {
-  // the caller's tiles the launch's tile covers: itself, or a block of merge_m x merge_n (fewer at the edges)
-  const bool merged = p.merge_m * p.merge_n > 1;
+  // the caller's tiles the launch's tile covers: itself, or (the MERGED builds, which only run launches whose
+  // tiles are blocks of the caller's) merge_m x merge_n of them, fewer at the edges.  A build of its own: the
+  // unmerged 256 x 256 kernel with these four scalars live across its K loop ran 4 % slower.
+  constexpr bool merged = MERGED;
   int first = tile_id, rows = 1, cols = 1, pm0 = 0, pn0 = 0;
-  if (merged) {
+  if constexpr (merged) {
     const TileCoord t = tile_map_fast(tile_id, p.num_pid_m, p.num_pid_n, p.G, p.tile_divs);
     pm0 = t.pid_m * p.merge_m;
     pn0 = t.pid_n * p.merge_n;
@@ -724,7 +730,7 @@ __device__ inline void publish_tile(const GemmKArgs& p, int tile_id, int lane) {
   }
   for (int i = 0; i < rows; ++i)
     for (int j = 0; j < cols; ++j) {
-      if (merged) first = tile_id_of(pm0 + i, pn0 + j, p.flag_num_pid_m, p.flag_num_pid_n, p.G);
+      if constexpr (merged) first = tile_id_of(pm0 + i, pn0 + j, p.flag_num_pid_m, p.flag_num_pid_n, p.G);
       IRIS_GLOBAL int32_t* own = (IRIS_GLOBAL int32_t*)(p.flags + first);
       for (int r = lane; r < p.ws; r += 64) {
         if (p.flag_mode == 2 && r == p.cur_rank) continue;
@@ -1156,9 +1162,10 @@ __device__ __attribute__((always_inline)) inline void big_tile_main(const GemmKA
 // (gemm_one_shot_all_reduce.py:197-271): store the partial tile, signal the
 // other ranks, wait for the tile's own flag, reduce it over all ranks and
 // store the result, tile by tile, while other programs are in their K loops.
-template <class Cfg, int OP, int ODT, bool SPLIT = false, bool FUSED = false>
+template <class Cfg, int OP, int ODT, bool SPLIT = false, bool FUSED = false, bool MERGED = false>
 __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(Cfg::WPE, Cfg::WPE))) void
 gemm_persistent_kernel(const GemmKArgs p) {
+  static_assert(!MERGED || (!SPLIT && !FUSED), "blocks of the caller's tiles: the plain build only");
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   IRIS_LDS char* lds = (IRIS_LDS char*)lds_raw;
   if constexpr (Cfg::IM * Cfg::IN * 4 > 128) {
@@ -1249,7 +1256,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       // a one-step tile: the previous tile has not been published yet
       IRIS_WAIT_VMCNT(0);
       __syncthreads();
-      if (wave == 0) publish_tile(p, pending_tile, lane);
+      if (wave == 0) publish_tile<MERGED>(p, pending_tile, lane);
       pending_tile = -1;
     }
     if constexpr (SPLIT) {
@@ -1293,7 +1300,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
           before = __builtin_amdgcn_readfirstlane(before);
           if (before == parts - 1) {
             // every slice is in memory: publish, and leave both counters at 0
-            if (p.flag_mode != 0) publish_tile(p, c_it.tile_id, lane);
+            if (p.flag_mode != 0) publish_tile<MERGED>(p, c_it.tile_id, lane);
             if (lane == 0) {
               flag_add_relaxed(done, -parts, false);
               flag_add_relaxed((IRIS_GLOBAL int32_t*)(p.locks + slot0), -parts, false);
@@ -1346,7 +1353,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
         __syncthreads();
         int ok = 1;
         if (p.ws > 1) {
-          if (wave == 0) publish_tile(p, c_it.tile_id, lane);  // +1 on every other rank (:207-218)
+          if (wave == 0) publish_tile<MERGED>(p, c_it.tile_id, lane);  // +1 on every other rank (:207-218)
           if (tid == 0) {
             *slot = wait_tile_flag((IRIS_GLOBAL int32_t*)(p.flags + c_it.tile_id), p.ws, p.sys != 0, p.timeout,
                                    p.status)
@@ -1378,7 +1385,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       } else if (p.flag_mode != 0) {
         IRIS_WAIT_VMCNT(0);  // this wave's stores of the tile have completed
         __syncthreads();
-        if (wave == 0) publish_tile(p, c_it.tile_id, lane);
+        if (wave == 0) publish_tile<MERGED>(p, c_it.tile_id, lane);
       }
       if (p.ts_end && tid == 0)
         __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + c_it.tile_id),
@@ -1522,7 +1529,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
         block_barrier_raw();
         if (pend >= 0) {
           if (skip == 0) {
-            if (wave == 0) publish_tile(p, pend, lane);
+            if (wave == 0) publish_tile<MERGED>(p, pend, lane);
             pending_tile = -1;
           } else {
             pending_skip = 0;
@@ -1614,7 +1621,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
   if (pending_tile >= 0) {
     IRIS_WAIT_VMCNT(0);
     __syncthreads();
-    if (wave == 0) publish_tile(p, pending_tile, lane);
+    if (wave == 0) publish_tile<MERGED>(p, pending_tile, lane);
   }
 }
 

@@ -253,6 +253,7 @@ void split_last_round(const iris_gemm_args& a, Plan* plan) {
   const GemmKernelEntry* e = plan->entry;
   plan->last_round = 0;
   if (!e || plan->skinny || plan->in_program || k.split_k != 1 || k.stream_k || k.sub_m != 1 || k.sub_n != 1) return;
+  if (k.merge_m * k.merge_n > 1) return;  // (the split-K build raises one flag per tile of its own)
   if (a.split_k != 0 || a.variant != 0 || a.mm_begin_timestamp || a.mm_end_timestamp) return;
   if (!a.partials || !a.locks || !e->splitk || !e->fn_split || k.num_sms != a.num_sms) return;
   if (a.num_sms > current_cu_count() || a.partials_slot_elems < (int64_t)e->cm * e->cn) return;
@@ -313,7 +314,7 @@ hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
     const hipError_t err = make_plan_body(b, &merged);
     // (only the persistent kernels, unsplit, publish merged tiles)
     if (err == hipSuccess && merged.entry && !merged.skinny && merged.k.split_k == 1 && !merged.k.stream_k &&
-        !merged.in_program) {
+        !merged.in_program && merged.entry->fn_merged) {
       *plan = merged;
       plan->k.merge_m = merge_m;
       plan->k.merge_n = merge_n;
@@ -588,6 +589,7 @@ namespace {
 GemmKernelFn plan_fn(const Plan& plan) {
   const GemmKernelEntry* e = plan.entry;
   if (plan.in_program) return e->fn_fused;
+  if (plan.k.merge_m * plan.k.merge_n > 1) return e->fn_merged;
   return (plan.k.split_k > 1 || plan.k.stream_k) ? e->fn_split : e->fn;
 }
 

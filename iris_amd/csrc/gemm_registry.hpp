@@ -23,6 +23,7 @@ struct GemmKernelEntry {
   GemmKernelFn fn;
   GemmKernelFn fn_split;  // split-K build, or null
   GemmKernelFn fn_fused;  // build with the one-shot reduce inside the program (store epilogues), or null
+  GemmKernelFn fn_merged;  // build whose tiles are blocks of the caller's (store epilogues, 256 x 128 and 256 x 256), or null
   const char* name;
 };
 
@@ -44,13 +45,26 @@ constexpr GemmKernelFn fused_fn() {
     return nullptr;
 }
 
+// The launcher only merges the caller's tiles into 256 x 128 and 256 x 256 ones, for the store epilogues, and
+// runs them with the table's first tile of either shape.
+template <class Cfg>
+constexpr bool merged_build = Cfg::CM == 256 && Cfg::DMA && Cfg::BK == 64 &&
+                              ((Cfg::CN == 256 && Cfg::LW == 0 && Cfg::NW == 8) || (Cfg::CN == 128 && Cfg::LW == 4));
+template <class Cfg, int OP, int ODT>
+constexpr GemmKernelFn merged_fn() {
+  if constexpr ((OP == OP_STORE16 || OP == OP_STORE32) && merged_build<Cfg>)
+    return &gemm_persistent_kernel<Cfg, OP, ODT, false, false, true>;
+  else
+    return nullptr;
+}
+
 template <class Cfg, int OP>
 constexpr GemmKernelEntry make_entry(const char* name) {
   constexpr int ODT = (OP == OP_STORE32 || OP == OP_ATOMIC32) ? IRIS_DTYPE_F32 : Cfg::DT;
   return GemmKernelEntry{Cfg::DT, OP,      Cfg::CM, Cfg::CN, Cfg::BK,        Cfg::WM,
                          Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::SPLIT_OWNER, Cfg::THREADS, Cfg::LW, Cfg::LDS_BYTES,
                          &gemm_persistent_kernel<Cfg, OP, ODT, false>, split_fn<Cfg, OP, ODT>(), fused_fn<Cfg, OP, ODT>(),
-                         name};
+                         merged_fn<Cfg, OP, ODT>(), name};
 }
 
 // The variants, in the launcher's order of preference: the first entry whose
@@ -122,6 +136,13 @@ constexpr GemmKernelEntry make_entry(const char* name) {
                                                   IRIS_GEMM_ODT(DT, OP), false, true>(const GemmKArgs);
 #define IRIS_GEMM_INSTANTIATE_FUSED_2(DT, OP, CM, CN, BK, WM, WN, S, DMA)
 #define IRIS_GEMM_INSTANTIATE_FUSED_4(DT, OP, CM, CN, BK, WM, WN, S, DMA)
+
+// the store epilogues' builds whose tiles are blocks of the caller's
+#define IRIS_GEMM_INSTANTIATE_MERGED(DT, OP)                                                                        \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 256, 64, 2, 4, 2, true, 0>, OP,                \
+                                                  IRIS_GEMM_ODT(DT, OP), false, false, true>(const GemmKArgs); \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 128, 64, 2, 2, 3, true, 4>, OP,                \
+                                                  IRIS_GEMM_ODT(DT, OP), false, false, true>(const GemmKArgs);
 
 #define IRIS_GEMM_DECLARE(TAG) const GemmKernelEntry* gemm_entries_##TAG(int* count);
 IRIS_GEMM_DECLARE(bf16_store16)
