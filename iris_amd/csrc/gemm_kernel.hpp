@@ -73,6 +73,16 @@ struct GemmKArgs {
   int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
   int sys;           // flag atomics at system scope (else agent)
   int vec_out;       // 16-byte vector access allowed on `out`
+  // > 0 (split-K launches with long parts; the value is total_tiles): the programs are numbered part by part
+  // rather than tile by tile, so that an XCD's programs walk the same range of K over neighbouring tiles and
+  // its L2 fetches each operand panel of that range once.  (Tile by tile, every program of an XCD walks a
+  // different range and nothing is shared: the operands then come from HBM once per tile.)
+  int part_major;
+  // The launch covers tiles tile_base .. tile_base + total_tiles - 1 of the num_pid_m x num_pid_n grid.  Only the
+  // split-K builds read it: a GEMM whose last round of tiles is split over the idle programs is an unsplit launch
+  // from tile 0 and a split one from tile_base.  (The unsplit 256 x 256 kernel with one more scalar live across
+  // its K loop ran 1.6 % slower on the headline shape.)
+  int tile_base;
   // Split-K: a tile's K-steps are shared out over `split_k` programs.  Part 0
   // owns the tile: the others leave their fp32 accumulators in `partials`
   // (slot = global item index, `partial_stride` floats apart) and raise
@@ -108,18 +118,8 @@ struct GemmKArgs {
   int cg_dt;         // element type of `cg`
   int fused_vec;     // 16-byte strips allowed on `out` and `cg` in the in-program reduce
 
-  // What only some builds read comes last, so that the others find every field where it was (the unsplit
-  // 256 x 256 kernel is sensitive to the scalars it keeps across its K loop).
-  // > 0 (split-K launches with long parts; the value is total_tiles): the programs are numbered part by part
-  // rather than tile by tile, so that an XCD's programs walk the same range of K over neighbouring tiles and
-  // its L2 fetches each operand panel of that range once.  (Tile by tile, every program of an XCD walks a
-  // different range and nothing is shared: the operands then come from HBM once per tile.)
-  int part_major;
-  // The launch covers tiles tile_base .. tile_base + total_tiles - 1 of the num_pid_m x num_pid_n grid.  Only the
-  // split-K builds read it: a GEMM whose last round of tiles is split over the idle programs is an unsplit launch
-  // from tile 0 and a split one from tile_base.  (The unsplit 256 x 256 kernel with one more scalar live across
-  // its K loop ran 1.6 % slower on the headline shape.)
-  int tile_base;
+  // (Last, and the two fields of the split-K builds above among theirs: nothing the unsplit kernels read has
+  // moved for them.  The unsplit 256 x 256 kernel is sensitive to where its arguments lie.)
   // merge_m * merge_n > 1: the launch's tiles (BM, BN, num_pid_m, num_pid_n, tile ids above) are merge_m x
   // merge_n of the caller's tiles; the flags stay the caller's, one per tile of BM / merge_m x BN / merge_n,
   // numbered over flag_num_pid_m x flag_num_pid_n tiles
@@ -715,7 +715,7 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
 // vector load and the increments leave together (one thread walking the ranks
 // waits for a scalar load per rank: 0.8 us for eight).
 template <bool MERGED = false>
-__device__ inline void publish_tile(const GemmKArgs& p, int tile_id, int lane) {
+__device__ __attribute__((always_inline)) inline void publish_tile(const GemmKArgs& p, int tile_id, int lane) {
   // the caller's tiles the launch's tile covers: itself, or (the MERGED builds, which only run launches whose
   // tiles are blocks of the caller's) merge_m x merge_n of them, fewer at the edges.  A build of its own: the
   // unmerged 256 x 256 kernel with these four scalars live across its K loop ran 4 % slower.

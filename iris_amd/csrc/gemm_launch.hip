@@ -524,13 +524,11 @@ hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan) {
   // A split launch of a 128-accumulator tile: the fetch state of the `_f4` build spills next
   // to the hand-over's registers ([128,4096] x [4096,1376] as one 256 x 128 tile row in 16
   // parts: 24.0 us against the plain tile's 21.2).
-  // (With 32 K-steps or more a part the spills are paid once and the K loop decides: [8192,12288] x
-  // [12288,512] as 128 tiles of 256 x 128 in two parts.)
-  {
-    const int nk = (a.K + pick->bk - 1) / pick->bk;
-    if (k.split_k != 1 && twin && !pick->split_owner && twin->bk == pick->bk && nk / k.split_k < 32)
-      plan->entry = twin;
-  }
+  // Where the compiler puts those spills changes with unrelated edits: [8192,12288] x [12288,512] as 128
+  // tiles of 256 x 128 in two parts has run in 131 us (none inside the K loop) and in 181 (one fragment
+  // spilled and reloaded every K-step) with the `_f4` build, 158 with the plain one, which is what every
+  // such launch takes.  (The second launch of a split last round runs the `_f4` build: HBM bounds it.)
+  if (k.split_k != 1 && twin && !pick->split_owner && twin->bk == pick->bk) plan->entry = twin;
   return hipSuccess;
 }
 
