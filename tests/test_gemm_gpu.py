@@ -748,6 +748,47 @@ def test_a_short_last_round_of_long_tiles_is_split_over_the_idle_programs(shmem,
                                                   4, ops.EPI_ALL_SCATTER, partials=partials, locks=locks)
 
 
+def test_split_last_round_with_the_one_shot_producer_and_reduce(shmem):
+    """K-shards on two ranks, 18 tiles of 256 x 64 on 16 programs, K = 8192 a rank:
+    each producer is two launches (16 whole tiles, then the last two in four
+    parts), the fp32 partials and the flags on the other rank are as from one
+    launch, and the reduce gives the oracle's sum."""
+    ws, M, N, dtype, grid = 2, 512, 576, torch.bfloat16, 16
+    K = 8192 * ws
+    A, B = make_ab(M, N, K, dtype, scale=0.01)
+    shards = O.k_shards(A, B, ws)
+    ah, bh = to_heap(shmem, A), to_heap(shmem, B)
+    kk = K // ws
+    part = shmem.zeros((M, N), dtype=torch.float32)
+    out = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, 256) * ops.cdiv(N, 64)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    partials, locks = split_workspace(shmem, grid, 256, 64)
+    hb = shmem.get_heap_bases()
+    for r in range(ws):
+        for t in (part, out, flags):
+            shmem.on_rank(t, r).zero_()
+    for r in range(ws):
+        args = (ah[:, r * kk:(r + 1) * kk], bh[r * kk:(r + 1) * kk, :], shmem.on_rank(part, r), shmem.on_rank(out, r),
+                shmem.on_rank(flags, r), hb, r, ws, grid, 256, 64, 64, 6, ops.EPI_ONE_SHOT)
+        kw = dict(phase=ops.PHASE_PRODUCE, partials=partials, locks=locks)
+        assert ops.gemm_plan_name(*args, **kw) == "256x64x64_w4x1_s3_f4+last_round_in_4_parts"
+        ops.gemm_launch(*args, **kw)
+        torch.cuda.synchronize()
+        assert int(locks.abs().max().item()) == 0
+        check_close(shmem.on_rank(part, r), O.shard_gemm(*shards[r], torch.float32), f"partial of rank {r}")
+    for r in range(ws):
+        assert shmem.on_rank(flags, r).cpu().tolist() == [ws - 1] * total
+    for r in range(ws):
+        ops.one_shot_reduce(shmem.on_rank(part, r), shmem.on_rank(out, r), shmem.on_rank(flags, r), hb, r, ws, 256, 64,
+                            6)
+    torch.cuda.synchronize()
+    want = O.one_shot_all_reduce(shards, torch.float32, dtype)
+    for r in range(ws):
+        check_close(shmem.on_rank(out, r), want, f"reduced on rank {r}")
+        assert not shmem.on_rank(flags, r).any()
+
+
 STREAM_K_CASES = [
     # M, N, K, BLK_M, BLK_N, grid, dtype
     (2048, 1376, 1024, 128, 128, 256, torch.bfloat16),  # 176 tiles x 16 steps on 256 programs: runs of 11
