@@ -187,7 +187,7 @@ struct GemmCfg {
   // stream-K runs hand over); the 128x64 wave tiles have no registers to spare
   // for that exchange and only take the sliced hand-over, in which a part's
   // accumulators are dead once its partial is written.
-  static constexpr bool SPLITK = DMA_ && KSUB % 2 == 0;
+  static constexpr bool SPLITK = DMA_ && KSUB % 2 == 0 && IM * IN * 4 <= 128;
   static constexpr bool SPLIT_OWNER = SPLITK && IM * IN * 4 <= 64;
   // Waves per SIMD the register budget is sized for: 256 registers a wave.
   static constexpr int WPE = IM * IN * 4 > 128 ? 1 : 2;
@@ -1156,6 +1156,216 @@ __device__ __attribute__((always_inline)) inline void big_tile_main(const GemmKA
   }
 }
 
+// The same tile with 64-deep stages and its prefetch staged in registers: whole 128-byte lines are fetched with
+// plain buffer loads into two sets of staging registers, a step and a half ahead and one load per block of
+// MFMAs over the whole step, and written into the LDS stage that the hand-over has just freed (two
+// ds_write_b128 per block of the step's second half).  The LDS layout is the DMA loader's, so the fragment
+// reads are the other tiles'.  The first two stages of a tile still come by LDS-DMA.
+template <class Cfg, int OP, int ODT>
+__device__ __attribute__((always_inline)) inline void big_tile_main_regs(const GemmKArgs& p, IRIS_LDS char* lds) {
+  static_assert(Cfg::DMA && Cfg::LW == 0 && Cfg::KSUB == 2 && Cfg::S == 2 && Cfg::IM == Cfg::IN && Cfg::IM == 8 &&
+                    Cfg::L == 16,
+                "register-staged K loop");
+  constexpr int L = Cfg::L;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  int pid;
+  if (p.xcd_per > 0) {
+    const int x = blockIdx.x % p.num_xcds, j = blockIdx.x / p.num_xcds;
+    pid = j < p.xcd_per ? x * p.xcd_per + j : p.num_sms * 2;
+  } else {
+    pid = xcd_remap(blockIdx.x, p.num_sms, p.num_xcds);
+  }
+  const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
+  const int n_mine = pid < p.total_tiles ? (p.total_tiles - pid + p.num_sms - 1) / p.num_sms : 0;
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  IRIS_LDS char* ws = lds + Cfg::S * Cfg::STAGE + wave * Cfg::WS_BYTES;
+  const int lrow = lane & 15, lq = lane >> 4;
+  const int swz = (lrow / Cfg::RP) % Cfg::CPR;
+  const int x0 = (lq ^ swz) * 16, x1 = ((4 + lq) ^ swz) * 16;  // the lane's chunk of the two substeps
+  const int a_row = (wm * Cfg::TM + lrow) * Cfg::BK * 2;
+  const int b_row = Cfg::A_BYTES + (wn * Cfg::TN + lrow) * Cfg::BK * 2;
+  const int wdst = wave * 1024 + lane * 16;  // where this lane's 16 bytes of load 0 land in a stage
+  const StreamRun sr{0, 0, 0};
+  Loader<Cfg> ld;
+  Frags<Cfg> fr;
+  f32x4 acc[Cfg::IM][Cfg::IN];
+  u32x4 stg[2][L];
+
+  // Load i of K-step k into registers (the DMA loader's addresses).  Written as an instruction of its own:
+  // the compiler, tracking a builtin's result across the loop's back edge, waits for every load in flight at
+  // the top of each iteration, which takes the prefetch away; the waits before the registers are used are
+  // counted by hand below instead (the loads complete in the order they were issued).
+  typedef int i32x4 __attribute__((ext_vector_type(4)));
+  i32x4 da = {0, 0, 0, 0}, db = {0, 0, 0, 0};  // buffer descriptors of the tile's A and B panels
+  auto fetch = [&](int k, int i) __attribute__((always_inline)) -> u32x4 {
+    const bool isA = i < Cfg::A_LOADS;
+    const int j = isA ? i : i - Cfg::A_LOADS;
+    const uint32_t off = isA ? ld.va + (uint32_t)(j * ld.step_a) : ld.vb + (uint32_t)(j * ld.step_b);
+    const int soff = k * Cfg::BK * 2;
+    u32x4 v;
+    if (isA)
+      asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(v) : "v"(off), "s"(da), "s"(soff) : "memory");
+    else
+      asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(v) : "v"(off), "s"(db), "s"(soff) : "memory");
+    return v;
+  };
+  auto descriptor = [&](const char* base, uint32_t bytes) __attribute__((always_inline)) -> i32x4 {
+    const uint64_t b = (uint64_t)base;
+    return i32x4{(int)(uint32_t)b, (int)(uint32_t)((b >> 32) & 0xFFFF), (int)bytes, 0x00020000};
+  };
+  // ... and from registers into its place in `stage`
+  auto put = [&](IRIS_LDS char* stage, int i, const u32x4& v) __attribute__((always_inline)) {
+    const bool isA = i < Cfg::A_LOADS;
+    const int j = isA ? i : i - Cfg::A_LOADS;
+    *reinterpret_cast<IRIS_LDS u32x4*>(stage + (isA ? 0 : Cfg::A_BYTES) + j * Cfg::NL * 1024 + wdst) = v;
+  };
+
+  // The first two steps of a tile on their way, by LDS-DMA into the two stages: issued before the previous
+  // tile's epilogue, so that they land under it.  (Step 2 goes into the first set of staging registers when the
+  // tile starts: registers that the compiler may spill around the epilogue must not have loads in flight,
+  // which it does not know of.)
+  auto start_tile = [&](const Item& nx) __attribute__((always_inline)) {
+    ld.setup(p, nx, wave, lane, 0);
+    {
+      // (the same panels and bounds as the loader's descriptors)
+      const int m0c = min(nx.m0, p.M - 1), n0c = min(nx.n0, p.N - 1);
+      const int rows_a = nx.m0 < p.M ? min(Cfg::CM, p.M - nx.m0) : 0, rows_b = nx.n0 < p.N ? min(Cfg::CN, p.N - nx.n0) : 0;
+      da = descriptor(p.a + (int64_t)m0c * p.sam * 2,
+                      rows_a > 0 ? (uint32_t)(((int64_t)(rows_a - 1) * p.sam + p.K) * 2) : 0);
+      db = descriptor(p.b + (int64_t)n0c * p.sbn * 2,
+                      rows_b > 0 ? (uint32_t)(((int64_t)(rows_b - 1) * p.sbn + p.K) * 2) : 0);
+    }
+    ld.issue(p, lds, 0, wave);
+    ld.before_step(1, wave, lane);
+    ld.issue(p, lds + Cfg::STAGE, 1, wave);
+    ld.before_step(2, wave, lane);
+  };
+  Item it;
+  if (n_mine > 0) {
+    it = decode_item<Cfg, false>(p, sr, pid, 0);
+    if (nk > 0) start_tile(it);
+  }
+  for (int t = 0; t < n_mine; ++t) {
+#pragma unroll
+    for (int i = 0; i < Cfg::IM; ++i)
+#pragma unroll
+      for (int j = 0; j < Cfg::IN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    Item nx = it;
+    if (nk > 0) {
+#pragma unroll
+      for (int i = 0; i < L; ++i) stg[0][i] = fetch(2, i);
+      // (a later tile's first two steps were waited for with the previous tile's stores)
+      if (t == 0) IRIS_WAIT_VMCNT(L);  // the DMA loads are older than the register loads
+      block_barrier_raw();
+      load_all<Cfg>(lds + a_row + x0, lds + b_row + x0, fr, 0);
+
+      // step g; W: the staging set that holds step g+2 (the other one takes step g+3)
+      auto step = [&](int g, auto w_tag) __attribute__((always_inline)) {
+        constexpr int W = decltype(w_tag)::value;
+        IRIS_LDS char* stage = lds + (g & 1) * Cfg::STAGE;
+        const IRIS_LDS char* nst = lds + ((g + 1) & 1) * Cfg::STAGE;
+        ld.before_step(g + 3, wave, lane);
+        // first half: multiply the first 32 of K, fetch the fragments of the second 32
+        // (memory instructions between the MFMAs of a block, not behind them: a wave that issues several
+        // in a row lets its matrix core run dry meanwhile)
+#pragma unroll
+        for (int i = 0; i < Cfg::IM; ++i) {
+#pragma unroll
+          for (int j = 0; j < Cfg::IN; ++j) {
+            Mfma<Cfg::DT>::run_acc(fr.b[0][j], fr.a[i], acc[i][j]);
+            if (j == 1) {
+              fr.b[1][i] = load_b<Cfg>(stage + b_row + x1, i);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+            if (j == 4) {
+              stg[W ^ 1][i] = fetch(g + 3, i);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
+          fr.a[i] = load_a<Cfg>(stage + a_row + x1, i);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        // second half: hand-over, then the next stage's first fragments, and stage g refilled from registers
+        mma_row<Cfg, false>(acc, fr, 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        IRIS_WAIT_LGKMCNT0();  // this wave's reads of stage g and its writes of stage g+1 are done
+        block_barrier_raw();
+        // Block i puts loads 2i and 2i+1 of step g+2, issued a step ago.  Younger than load 2i+1 are the
+        // 14 - 2i that followed it then, this step's first eight and the i of its second half so far.
+        auto second_half = [&](auto ic) __attribute__((always_inline)) {
+          constexpr int i = decltype(ic)::value;
+          if constexpr (i == 0) {
+            fr.a[i] = load_a<Cfg>(nst + a_row + x0, i);
+            fr.b[0][i] = load_b<Cfg>(nst + b_row + x0, i);
+            IRIS_WAIT_VMCNT(22 - i);
+            put(stage, 2 * i, stg[W][2 * i]);
+            put(stage, 2 * i + 1, stg[W][2 * i + 1]);
+            stg[W ^ 1][Cfg::IM + i] = fetch(g + 3, Cfg::IM + i);
+            __builtin_amdgcn_sched_barrier(0);
+          } else {
+#pragma unroll
+            for (int j = 0; j < Cfg::IN; ++j) {
+              Mfma<Cfg::DT>::run_acc(fr.b[1][j], fr.a[i], acc[i][j]);
+              if (j == 1) {
+                fr.b[0][i] = load_b<Cfg>(nst + b_row + x0, i);
+                __builtin_amdgcn_sched_barrier(0);
+              }
+              if (j == 3) {
+                IRIS_WAIT_VMCNT(22 - i);
+                put(stage, 2 * i, stg[W][2 * i]);
+                __builtin_amdgcn_sched_barrier(0);
+              }
+              if (j == 5) {
+                put(stage, 2 * i + 1, stg[W][2 * i + 1]);
+                __builtin_amdgcn_sched_barrier(0);
+              }
+              if (j == 6) {
+                stg[W ^ 1][Cfg::IM + i] = fetch(g + 3, Cfg::IM + i);
+                __builtin_amdgcn_sched_barrier(0);
+              }
+            }
+            fr.a[i] = load_a<Cfg>(nst + a_row + x0, i);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        };
+        second_half(std::integral_constant<int, 0>{});
+        second_half(std::integral_constant<int, 1>{});
+        second_half(std::integral_constant<int, 2>{});
+        second_half(std::integral_constant<int, 3>{});
+        second_half(std::integral_constant<int, 4>{});
+        second_half(std::integral_constant<int, 5>{});
+        second_half(std::integral_constant<int, 6>{});
+        second_half(std::integral_constant<int, 7>{});
+      };
+      int g = 0;
+      for (; g + 1 < nk; g += 2) {
+        step(g, std::integral_constant<int, 0>{});
+        step(g + 1, std::integral_constant<int, 1>{});
+      }
+      if (g < nk) step(g, std::integral_constant<int, 0>{});
+      // every wave is done with the stages (its reads, and its writes of the steps past the last, which are
+      // zeros): the next tile's first loads may go
+      IRIS_WAIT_LGKMCNT0();
+      block_barrier_raw();
+      if (t + 1 < n_mine) {
+        nx = decode_item<Cfg, false>(p, sr, pid, t + 1);
+        start_tile(nx);
+      }
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    } else if (t + 1 < n_mine) {
+      nx = decode_item<Cfg, false>(p, sr, pid, t + 1);
+    }
+    store_acc<Cfg, OP, ODT>(p, acc, ws, it.m0 + wm * Cfg::TM, it.n0 + wn * Cfg::TN, it.m_end, it.n_end, lane);
+    IRIS_WAIT_VMCNT(0);
+    IRIS_WAIT_LGKMCNT0();
+    __syncthreads();
+    if (p.flag_mode != 0 && wave == 0) publish_tile(p, it.tile_id, lane);
+    it = nx;
+  }
+}
+
 // SPLIT: the split-K build of the kernel (only launched with p.split_k > 1);
 // the plain build carries none of its code or state.
 // FUSED: the one-shot epilogue as the reference program runs it
@@ -1170,7 +1380,12 @@ gemm_persistent_kernel(const GemmKArgs p) {
   IRIS_LDS char* lds = (IRIS_LDS char*)lds_raw;
   if constexpr (Cfg::IM * Cfg::IN * 4 > 128) {
     static_assert(!SPLIT, "the 256-accumulator tiles have no split-K build");
-    if constexpr (!FUSED) big_tile_main<Cfg, OP, ODT>(p, lds);  // (no build with the reduce inside either)
+    if constexpr (!FUSED) {  // (no build with the reduce inside either)
+      if constexpr (Cfg::KSUB == 2)
+        big_tile_main_regs<Cfg, OP, ODT>(p, lds);
+      else
+        big_tile_main<Cfg, OP, ODT>(p, lds);
+    }
     return;
   }
 

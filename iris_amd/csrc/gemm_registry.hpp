@@ -108,7 +108,8 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   X(DT, OP, 128, 128, 32, 2, 2, 4, true, 0, 0, "128x128x32_w2x2_s4")         \
   X(DT, OP, 64, 64, 64, 2, 2, 4, true, 4, 1, "64x64x64_w2x2_s4_f4")          \
   X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")        \
-  X(DT, OP, 256, 256, 32, 2, 2, 4, true, 0, 0, "256x256x32_w2x2_s4")
+  X(DT, OP, 256, 256, 32, 2, 2, 4, true, 0, 0, "256x256x32_w2x2_s4")         \
+  X(DT, OP, 256, 256, 64, 2, 2, 2, true, 0, 0, "256x256x64_w2x2_s2_regs")
 
 #define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, SPLIT, NAME) \
   make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP>(NAME),
