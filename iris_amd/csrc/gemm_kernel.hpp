@@ -1288,7 +1288,10 @@ __device__ __attribute__((always_inline)) inline void big_tile_main_regs(const G
           __builtin_amdgcn_sched_barrier(0);
         }
         // second half: hand-over, then the next stage's first fragments, and stage g refilled from registers
-        mma_row<Cfg, false>(acc, fr, 1, 0);
+        // (half of the first block's MFMAs cover the wait and the barrier, the other half the memory
+        // instructions right behind it)
+#pragma unroll
+        for (int j = 0; j < Cfg::IN / 2; ++j) Mfma<Cfg::DT>::run_acc(fr.b[1][j], fr.a[0], acc[0][j]);
         __builtin_amdgcn_sched_barrier(0);
         IRIS_WAIT_LGKMCNT0();  // this wave's reads of stage g and its writes of stage g+1 are done
         block_barrier_raw();
@@ -1297,12 +1300,20 @@ __device__ __attribute__((always_inline)) inline void big_tile_main_regs(const G
         auto second_half = [&](auto ic) __attribute__((always_inline)) {
           constexpr int i = decltype(ic)::value;
           if constexpr (i == 0) {
-            fr.a[i] = load_a<Cfg>(nst + a_row + x0, i);
             fr.b[0][i] = load_b<Cfg>(nst + b_row + x0, i);
+            __builtin_amdgcn_sched_barrier(0);
+            Mfma<Cfg::DT>::run_acc(fr.b[1][4], fr.a[0], acc[0][4]);
             IRIS_WAIT_VMCNT(22 - i);
             put(stage, 2 * i, stg[W][2 * i]);
+            __builtin_amdgcn_sched_barrier(0);
+            Mfma<Cfg::DT>::run_acc(fr.b[1][5], fr.a[0], acc[0][5]);
             put(stage, 2 * i + 1, stg[W][2 * i + 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            Mfma<Cfg::DT>::run_acc(fr.b[1][6], fr.a[0], acc[0][6]);
             stg[W ^ 1][Cfg::IM + i] = fetch(g + 3, Cfg::IM + i);
+            __builtin_amdgcn_sched_barrier(0);
+            Mfma<Cfg::DT>::run_acc(fr.b[1][7], fr.a[0], acc[0][7]);
+            fr.a[i] = load_a<Cfg>(nst + a_row + x0, i);
             __builtin_amdgcn_sched_barrier(0);
           } else {
 #pragma unroll
