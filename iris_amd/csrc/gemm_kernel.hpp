@@ -168,7 +168,9 @@ struct GemmCfg {
   static constexpr int DT = DT_, CM = CM_, CN = CN_, BK = BK_, WM = WM_, WN = WN_, S = S_;
   static constexpr bool DMA = DMA_;
   static constexpr int NW = WM * WN, NT = NW * 64;  // the waves (threads) that multiply and store
-  static constexpr int LW = LW_;
+  // LW_ == 1 marks the four-wave 256 x 256 tile whose stages are refilled by LDS-DMA (no wave only fetches)
+  static constexpr bool BIG_DMA = LW_ == 1;
+  static constexpr int LW = BIG_DMA ? 0 : LW_;
   static constexpr int NL = LW ? LW : NW;           // the waves that fetch
   static constexpr int THREADS = (NW + LW) * 64;    // launch size
   static constexpr int TM = CM / WM, TN = CN / WN;
@@ -1254,10 +1256,12 @@ __device__ __attribute__((always_inline)) inline void big_tile_main_regs(const G
       for (int j = 0; j < Cfg::IN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     Item nx = it;
     if (nk > 0) {
+      if constexpr (!Cfg::BIG_DMA) {
 #pragma unroll
-      for (int i = 0; i < L; ++i) stg[0][i] = fetch(2, i);
+        for (int i = 0; i < L; ++i) stg[0][i] = fetch(2, i);
+      }
       // (a later tile's first two steps were waited for with the previous tile's stores)
-      if (t == 0) IRIS_WAIT_VMCNT(L);  // the DMA loads are older than the register loads
+      if (t == 0) IRIS_WAIT_VMCNT(Cfg::BIG_DMA ? 0 : L);  // the DMA loads are older than the register loads
       block_barrier_raw();
       load_all<Cfg>(lds + a_row + x0, lds + b_row + x0, fr, 0);
 
@@ -1266,7 +1270,7 @@ __device__ __attribute__((always_inline)) inline void big_tile_main_regs(const G
         constexpr int W = decltype(w_tag)::value;
         IRIS_LDS char* stage = lds + (g & 1) * Cfg::STAGE;
         const IRIS_LDS char* nst = lds + ((g + 1) & 1) * Cfg::STAGE;
-        ld.before_step(g + 3, wave, lane);
+        ld.before_step(Cfg::BIG_DMA ? g + 2 : g + 3, wave, lane);
         // first half: multiply the first 32 of K, fetch the fragments of the second 32
         // (memory instructions between the MFMAs of a block, not behind them: a wave that issues several
         // in a row lets its matrix core run dry meanwhile)
@@ -1279,7 +1283,7 @@ __device__ __attribute__((always_inline)) inline void big_tile_main_regs(const G
               fr.b[1][i] = load_b<Cfg>(stage + b_row + x1, i);
               __builtin_amdgcn_sched_barrier(0);
             }
-            if (j == 4) {
+            if (j == 4 && !Cfg::BIG_DMA) {
               stg[W ^ 1][i] = fetch(g + 3, i);
               __builtin_amdgcn_sched_barrier(0);
             }
@@ -1294,6 +1298,7 @@ __device__ __attribute__((always_inline)) inline void big_tile_main_regs(const G
         for (int j = 0; j < Cfg::IN / 2; ++j) Mfma<Cfg::DT>::run_acc(fr.b[1][j], fr.a[0], acc[0][j]);
         __builtin_amdgcn_sched_barrier(0);
         IRIS_WAIT_LGKMCNT0();  // this wave's reads of stage g and its writes of stage g+1 are done
+        if constexpr (Cfg::BIG_DMA) IRIS_WAIT_VMCNT(0);  // its part of stage g+1 has landed
         block_barrier_raw();
         // Block i puts loads 2i and 2i+1 of step g+2, issued a step ago.  Younger than load 2i+1 are the
         // 14 - 2i that followed it then, this step's first eight and the i of its second half so far.
@@ -1303,14 +1308,21 @@ __device__ __attribute__((always_inline)) inline void big_tile_main_regs(const G
             fr.b[0][i] = load_b<Cfg>(nst + b_row + x0, i);
             __builtin_amdgcn_sched_barrier(0);
             Mfma<Cfg::DT>::run_acc(fr.b[1][4], fr.a[0], acc[0][4]);
-            IRIS_WAIT_VMCNT(22 - i);
-            put(stage, 2 * i, stg[W][2 * i]);
+            if constexpr (Cfg::BIG_DMA) {
+              ld.issue_at(p, stage, g + 2, wave, 2 * i);
+            } else {
+              IRIS_WAIT_VMCNT(22 - i);
+              put(stage, 2 * i, stg[W][2 * i]);
+            }
             __builtin_amdgcn_sched_barrier(0);
             Mfma<Cfg::DT>::run_acc(fr.b[1][5], fr.a[0], acc[0][5]);
-            put(stage, 2 * i + 1, stg[W][2 * i + 1]);
+            if constexpr (Cfg::BIG_DMA)
+              ld.issue_at(p, stage, g + 2, wave, 2 * i + 1);
+            else
+              put(stage, 2 * i + 1, stg[W][2 * i + 1]);
             __builtin_amdgcn_sched_barrier(0);
             Mfma<Cfg::DT>::run_acc(fr.b[1][6], fr.a[0], acc[0][6]);
-            stg[W ^ 1][Cfg::IM + i] = fetch(g + 3, Cfg::IM + i);
+            if constexpr (!Cfg::BIG_DMA) stg[W ^ 1][Cfg::IM + i] = fetch(g + 3, Cfg::IM + i);
             __builtin_amdgcn_sched_barrier(0);
             Mfma<Cfg::DT>::run_acc(fr.b[1][7], fr.a[0], acc[0][7]);
             fr.a[i] = load_a<Cfg>(nst + a_row + x0, i);
@@ -1324,15 +1336,22 @@ __device__ __attribute__((always_inline)) inline void big_tile_main_regs(const G
                 __builtin_amdgcn_sched_barrier(0);
               }
               if (j == 3) {
-                IRIS_WAIT_VMCNT(22 - i);
-                put(stage, 2 * i, stg[W][2 * i]);
+                if constexpr (Cfg::BIG_DMA) {
+                  ld.issue_at(p, stage, g + 2, wave, 2 * i);
+                } else {
+                  IRIS_WAIT_VMCNT(22 - i);
+                  put(stage, 2 * i, stg[W][2 * i]);
+                }
                 __builtin_amdgcn_sched_barrier(0);
               }
               if (j == 5) {
-                put(stage, 2 * i + 1, stg[W][2 * i + 1]);
+                if constexpr (Cfg::BIG_DMA)
+                  ld.issue_at(p, stage, g + 2, wave, 2 * i + 1);
+                else
+                  put(stage, 2 * i + 1, stg[W][2 * i + 1]);
                 __builtin_amdgcn_sched_barrier(0);
               }
-              if (j == 6) {
+              if (j == 6 && !Cfg::BIG_DMA) {
                 stg[W ^ 1][Cfg::IM + i] = fetch(g + 3, Cfg::IM + i);
                 __builtin_amdgcn_sched_barrier(0);
               }

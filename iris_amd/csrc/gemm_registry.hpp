@@ -109,7 +109,8 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   X(DT, OP, 64, 64, 64, 2, 2, 4, true, 4, 1, "64x64x64_w2x2_s4_f4")          \
   X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")        \
   X(DT, OP, 256, 256, 32, 2, 2, 4, true, 0, 0, "256x256x32_w2x2_s4")         \
-  X(DT, OP, 256, 256, 64, 2, 2, 2, true, 0, 0, "256x256x64_w2x2_s2_regs")
+  X(DT, OP, 256, 256, 64, 2, 2, 2, true, 0, 0, "256x256x64_w2x2_s2_regs")    \
+  X(DT, OP, 256, 256, 64, 2, 2, 2, true, 1, 0, "256x256x64_w2x2_s2_dma")
 
 #define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, SPLIT, NAME) \
   make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP>(NAME),
@@ -135,6 +136,7 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 #define IRIS_GEMM_INSTANTIATE_FUSED_0(DT, OP, CM, CN, BK, WM, WN, S, DMA)                     \
   template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP, \
                                                   IRIS_GEMM_ODT(DT, OP), false, true>(const GemmKArgs);
+#define IRIS_GEMM_INSTANTIATE_FUSED_1(DT, OP, CM, CN, BK, WM, WN, S, DMA)
 #define IRIS_GEMM_INSTANTIATE_FUSED_2(DT, OP, CM, CN, BK, WM, WN, S, DMA)
 #define IRIS_GEMM_INSTANTIATE_FUSED_4(DT, OP, CM, CN, BK, WM, WN, S, DMA)
 
