@@ -71,7 +71,7 @@ def test_one_shot_consumer_polls_while_producers_publish(shmem, two_streams, ws,
     M = N = 4096
     K, BM, BN, G = 2048, 128, 128, 6
     dtype = torch.bfloat16
-    A, B = make_ab(M, N, K * ws, dtype, scale=0.05, seed=ws * 10 + variant)
+    A, B = make_ab(M, N, K * ws, dtype, seed=ws * 10 + variant)
     a_full, b_full = to_heap(shmem, A), to_heap(shmem, B)
     c = shmem.zeros((M, N), dtype=torch.float32)
     cg = shmem.zeros((M, N), dtype=dtype)
@@ -141,7 +141,7 @@ def test_scatter_ready_flags_gate_a_concurrent_reader(shmem, two_streams, scope)
     flag is up.  Both copies hold the same tile, so the sum is exactly twice it."""
     ws, M, NL, K, BM, BN, G = 2, 4096, 2048, 2048, 128, 128, 4
     dtype = torch.bfloat16
-    A, B = make_ab(M, NL, K, dtype, scale=0.05, seed=5)
+    A, B = make_ab(M, NL, K, dtype, seed=5)
     a, b = to_heap(shmem, A), to_heap(shmem, B)
     cg = shmem.zeros((M, NL * ws), dtype=dtype)
     out = shmem.zeros((M, NL), dtype=torch.float32)
@@ -207,7 +207,7 @@ def test_one_shot_inside_the_program_two_ranks_side_by_side(shmem, two_streams, 
     128 programs each share the 256 CUs, one stream per rank."""
     ws, G = 2, 6
     dtype = torch.bfloat16
-    A, B = make_ab(M, N, K * ws, dtype, scale=0.05, seed=M + N)
+    A, B = make_ab(M, N, K * ws, dtype, seed=M + N)
     a_full, b_full = to_heap(shmem, A), to_heap(shmem, B)
     c = shmem.zeros((M, N), dtype=partial_dtype)
     cg = shmem.zeros((M, N), dtype=dtype)

@@ -96,7 +96,7 @@ def test_33_to_64_rows_other_epilogues_and_the_launcher_choice(shmem):
     """fp32 partial with the one-shot signal on 4 virtual ranks, atomic add; and
     when the launch stays with the persistent kernels."""
     ws, M, N, K, dtype = 4, 40, 384, 4 * 2048, torch.bfloat16
-    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    A, B = make_ab(M, N, K, dtype)
     shards = O.k_shards(A, B, ws)
     ah, bh = to_heap(shmem, A), to_heap(shmem, B)
     kk = K // ws
@@ -203,7 +203,7 @@ def test_one_shot_producer_and_reduce(shmem, pdtype):
     """K-split over 4 ranks: each rank's partial through the few-rows kernel,
     +1 on every other rank's flag per tile, then the reduce kernel."""
     ws, M, N, K, BM, BN, G, dtype = 4, 16, 384, 4 * 256, 32, 128, 6, torch.bfloat16
-    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    A, B = make_ab(M, N, K, dtype)
     shards = O.k_shards(A, B, ws)
     ah, bh = to_heap(shmem, A), to_heap(shmem, B)
     kk = K // ws
@@ -246,7 +246,7 @@ def test_one_shot_fused_phase(shmem, ws, phase):
     then the last rank runs both phases."""
     M, N, BM, BN, G, dtype = 9, 272, 16, 64, 3, torch.bfloat16
     K = 192 * ws
-    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    A, B = make_ab(M, N, K, dtype)
     shards = O.k_shards(A, B, ws)
     ah, bh = to_heap(shmem, A), to_heap(shmem, B)
     kk = K // ws
@@ -279,7 +279,7 @@ def test_one_shot_fused_phase(shmem, ws, phase):
 def test_atomic_accumulate_of_k_shards(shmem, M, out_dtype):
     """08 epilogue: every rank adds its K-shard product into every rank's C."""
     ws, N, K, BM, BN, dtype = 4, 208, 4 * 320, 32, 64, torch.bfloat16
-    A, B = make_ab(M, N, K, dtype, scale=0.05)
+    A, B = make_ab(M, N, K, dtype)
     shards = O.k_shards(A, B, ws)
     ah, bh = to_heap(shmem, A), to_heap(shmem, B)
     kk = K // ws
