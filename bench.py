@@ -216,7 +216,7 @@ def context_figures(a, b, c_global, flops, gemm_on):
     """
     import torch
 
-    from iris_amd import ops
+    from iris_amd import ops, testing
 
     out = {}
     ms = steady_ms(lambda: torch.matmul(a, b, out=c_global))
@@ -237,8 +237,8 @@ def context_figures(a, b, c_global, flops, gemm_on):
     sink = torch.empty(groups * 512, dtype=torch.float32, device="cuda")
     for name, operands in (("random N(0,0.02)", (torch.randn(32768, device="cuda") * 0.02).to(torch.bfloat16)),
                            ("zeros", torch.zeros(32768, dtype=torch.bfloat16, device="cuda"))):
-        fl = ops.mfma_probe(operands, sink, iters, groups)
-        ms = steady_ms(lambda: ops.mfma_probe(operands, sink, iters, groups), n=100)
+        fl = testing.mfma_probe(operands, sink, iters, groups)
+        ms = steady_ms(lambda: testing.mfma_probe(operands, sink, iters, groups), n=100)
         out[f"mfma_sustained[{name}]"] = {"what": "register-only v_mfma_f32_16x16x32_bf16 loop, 8 waves per CU",
                                            "tflops": round(fl / (ms * 1e-3) / 1e12, 1)}
         # what the output stores of the headline launch cost next to the matrix cores, and whether spreading
@@ -248,7 +248,7 @@ def context_figures(a, b, c_global, flops, gemm_on):
         region = torch.empty(tiles * groups * 131072, dtype=torch.uint8, device="cuda")
         t = {}
         for label, chunk in (("none", 0), ("tile_at_once", 16), ("one_store_per_k_step", 1)):
-            t[label] = steady_ms(lambda: ops.store_probe(operands, sink, region, tiles, chunk, groups), n=100) * 1e3
+            t[label] = steady_ms(lambda: testing.store_probe(operands, sink, region, tiles, chunk, groups), n=100) * 1e3
         out[f"store_cost[{name}]"] = {
             "what": "register-only MFMAs of 4 tiles a CU + 128 MiB of write-through stores (16 one-KiB stores a wave "
                     "and tile), us per launch",

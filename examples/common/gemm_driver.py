@@ -74,7 +74,9 @@ def parse_args(defaults, argv=None):
     parser.add_argument("--waves_per_eu", type=int, default=0, help="Waves per execution unit")
     parser.add_argument("--mfmaInstrSize", type=int, default=16, help="MFMA instruction size")
     parser.add_argument("--kpack", type=int, default=defaults["kpack"], help="K packing size")
-    parser.add_argument("--heap_size", type=int, default=1 << 33, help="Iris heap size")
+    parser.add_argument("--heap_size", type=int, default=None,
+                        help="Iris heap size (default: 1 << 33; with one process per rank, whose heaps are mapped "
+                             "through IPC, the largest size such a mapping takes here, just under 2 GiB)")
     parser.add_argument("--gemm_sms", type=int, default=256, help="Number of persistent programs")
     parser.add_argument("--total_sms", type=int, default=304, help="Total number of SMs")
     parser.add_argument("--virtual_ranks", type=int, default=1, help="Ranks played by this one GPU")
@@ -89,6 +91,14 @@ def main(algorithm, argv=None):
 
     ranks = args["virtual_ranks"]
     # one process per rank when a launcher's environment says so, else this process plays `ranks` ranks
+    if args["heap_size"] is None:
+        args["heap_size"] = 1 << 33  # the reference scripts' default (benchmark.py:67)
+        if ranks == 1 and iris.launched_as_ranks():
+            # peers map this heap through IPC, which takes less than 2 GiB per mapping here; only a size the
+            # user asked for is an error
+            args["heap_size"] = iris.IPC_MAX_HEAP_BYTES
+            print(f"[Iris] heap_size defaults to {args['heap_size']} bytes with one process per rank "
+                  "(IPC mappings stay under 2 GiB)")
     shmem = iris.iris(args["heap_size"], virtual_ranks=ranks) if ranks > 1 else iris.iris(args["heap_size"])
     rank = shmem.get_rank()
     world_size = shmem.get_num_ranks()
@@ -97,8 +107,10 @@ def main(algorithm, argv=None):
     played = [rank] if multi_process else list(range(world_size))
     if multi_process:
         matmul.scope = ops.SCOPE_SYSTEM  # peers are other processes (the reference's scope="sys")
-    if multi_process and algorithm == "one_shot_all_reduce" and iris._hip.count_devices() < world_size:
-        # ranks that share a GPU wait for each other's programs on it: all of them must fit at once
+    if multi_process and iris._hip.count_devices() < world_size:
+        # Ranks that share a GPU: programs wait for programs (09 for the peers' tiles, 07 / 08 for the other
+        # parts of a tile whose K range the launcher has shared out), so every rank's whole grid must fit the
+        # device at once.
         fit = max(8, (cu_count // world_size) // 8 * 8)
         if args["gemm_sms"] > fit:
             shmem.log(f"gemm_sms {args['gemm_sms']} -> {fit}: {world_size} ranks share the {cu_count} CUs of one GPU")

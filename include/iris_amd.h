@@ -74,7 +74,7 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 #define IRIS_DTYPE_F32 0
 #define IRIS_DTYPE_F16 1
 #define IRIS_DTYPE_BF16 2
-/* integer element types: only iris_rma_selftest_launch and iris_p2p_bench_launch take them */
+/* integer element types: only iris_p2p_bench_launch (and the unit-test kernels of iris_amd_testing.h) take them */
 #define IRIS_DTYPE_I8 3
 #define IRIS_DTYPE_I16 4
 #define IRIS_DTYPE_I32 5
@@ -96,7 +96,19 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 /* flag scopes */
 #define IRIS_SCOPE_AGENT 0  /* all "ranks" live on this GPU */
 #define IRIS_SCOPE_SYSTEM 1 /* the reference's scope="sys" */
-#define IRIS_SCOPE_WORKGROUP 2 /* scope="cta"; only iris_rma_selftest_launch takes it */
+#define IRIS_SCOPE_WORKGROUP 2 /* scope="cta"; only the unit-test kernels of iris_amd_testing.h take it */
+
+/* How a tile's flag orders the tile's data (iris_gemm_args.flag_sem, iris_reduce_args.flag_sem).
+ * WRITE_THROUGH (the default): the tile is stored with write-through stores at the flags' scope, the producer
+ * waits for their acknowledgement and raises the flag with a relaxed atomic; the consumer polls relaxed and reads
+ * with loads that are coherent at that scope.  No cache write-back and no invalidate per tile.  This scheme has
+ * been validated with producers and consumers running side by side on ONE device (at both scopes); it has not
+ * been run across devices.
+ * RELEASE_ACQUIRE: the reference's semantics verbatim -- atomic_add(flag, 1, sem="release") on the producer
+ * side, sem="acquire" on the consumer's wait (gemm_one_shot_all_reduce.py:207-234).  What a launch across
+ * devices should use until the default has been validated there; costs an L2 write-back per published tile. */
+#define IRIS_FLAG_SEM_WRITE_THROUGH 0
+#define IRIS_FLAG_SEM_RELEASE_ACQUIRE 1
 
 /* status word values (max-reduced by the kernels into *status) */
 #define IRIS_STATUS_OK 0
@@ -178,6 +190,7 @@ typedef struct iris_gemm_args {
    * its share of the tile's rows.  Both add the partials in part order: the
    * results are bit-identical. */
   int32_t split_handover;
+  int32_t flag_sem;     /* IRIS_FLAG_SEM_*: how a tile's flag orders its data                    */
 } iris_gemm_args;
 
 /*
@@ -262,6 +275,7 @@ typedef struct iris_reduce_args {
   int32_t wait_flags; /* 0: skip the flag wait (plain P-way sum) */
   int32_t variant;
   uint64_t spin_timeout_ticks;
+  int32_t flag_sem;   /* IRIS_FLAG_SEM_*: RELEASE_ACQUIRE adds an acquire fence after every flag wait */
 } iris_reduce_args;
 
 int iris_one_shot_reduce_launch(const iris_reduce_args* args, void* stream);
@@ -301,66 +315,6 @@ void iris_tile_map_host(int32_t tile_id, int32_t M, int32_t N, int32_t block_m, 
  */
 int iris_stream_k_schedule_host(int32_t total_tiles, int32_t k_steps, int32_t num_programs, int32_t pid,
                                 int32_t* items, int32_t cap, int32_t* n_items);
-
-/*
- * Measurement aid; no counterpart in the reference.  `num_groups` workgroups of
- * 8 waves each run `iters` rounds of 16 v_mfma_f32_16x16x32 (ab_dtype: F16 or
- * BF16) per wave on operands read once from `operands` (64 KiB, 16-byte
- * aligned, any bit patterns), with nothing but registers inside the loop:
- * num_groups * 8 * iters * 16 * 16384 FLOP per launch.  `sink` receives one
- * float per thread (num_groups * 512).  Timed by the caller, it gives the rate
- * the matrix cores sustain on such data under the board's power limit.
- */
-int iris_mfma_probe_launch(const void* operands, float* sink, int32_t ab_dtype, int32_t iters, int32_t num_groups,
-                           void* stream);
-
-/*
- * Measurement aid; no counterpart in the reference.  What a tile's worth of
- * output stores costs next to the matrix cores, by how the stores are spread:
- * each of `num_groups` workgroups of 8 waves runs `tiles` tiles, a tile being
- * 16 K-steps of 64 register-only bf16 MFMAs a wave (a 256 x 256 x 1024 tile's
- * worth) and 16 one-KiB stores a wave (128 KiB a group) to a region of its own
- * in `out` (`out_bytes` >= num_groups * 128 KiB, 16-byte aligned; tile t goes
- * to offset t * num_groups * 128 KiB modulo what fits).  `chunk` stores go out
- * back to back every `chunk` K-steps: 16 = a whole tile at once, 4, 1 = one a
- * K-step, 0 = none.  `write_through`: sc1 stores (else plain); `lockstep`: the
- * waves of a group meet at a barrier after every K-step.  `operands` and
- * `sink` as for iris_mfma_probe_launch.
- */
-int iris_store_probe_launch(const void* operands, float* sink, void* out, uint64_t out_bytes, int32_t tiles,
-                            int32_t chunk, int32_t write_through, int32_t lockstep, int32_t num_groups, void* stream);
-
-/*
- * Device-side remote access (include/iris_device.hpp, the HIP counterpart of
- * iris/iris.py:317-521) exercised the way the reference's unit tests exercise
- * the Triton functions: one workgroup, lane i < block_size owns element i of
- * `data` / `results` (buffers at the same heap offset on every rank), and every
- * rank 0..num_ranks-1 is the target in turn.
- *   LOAD        results[i]  = sum over ranks of load(data + i)      tests/unittests/test_load.py:8-31
- *   STORE       store(results + i, data[i]) on every rank           tests/unittests/test_store.py:8-30
- *   GET         get(data + i -> results + i), accumulate, store     tests/unittests/test_get.py:8-31
- *   PUT         put(data + i -> results + i) on every rank          tests/unittests/test_put.py:8-26
- *   ATOMIC_ADD  atomic_add(results + i, 1) on every rank            tests/unittests/test_atomic_add.py:8-30
- *   ATOMIC_SUB  atomic_sub(results + i, 1) on every rank            (iris/iris.py:452-473; no reference test)
- *   ATOMIC_CAS  atomic_cas(results, 0 -> num_ranks) on every rank   tests/unittests/test_atomic_cas.py:8-24
- *   ATOMIC_XCHG atomic_xchg(results, num_ranks) on every rank       tests/unittests/test_atomic_xchg.py:8-23
- * sem / scope only matter for the atomics.  block_size is 1..64; int8 has no atomics.
- */
-#define IRIS_RMA_LOAD 0
-#define IRIS_RMA_STORE 1
-#define IRIS_RMA_GET 2
-#define IRIS_RMA_PUT 3
-#define IRIS_RMA_ATOMIC_ADD 4
-#define IRIS_RMA_ATOMIC_SUB 5
-#define IRIS_RMA_ATOMIC_CAS 6
-#define IRIS_RMA_ATOMIC_XCHG 7
-#define IRIS_SEM_RELAXED 0
-#define IRIS_SEM_ACQUIRE 1
-#define IRIS_SEM_RELEASE 2
-#define IRIS_SEM_ACQ_REL 3
-int iris_rma_selftest_launch(int32_t op, int32_t dtype, int32_t sem, int32_t scope, const void* data, void* results,
-                             const uint64_t* heap_bases, int32_t cur_rank, int32_t num_ranks, int32_t block_size,
-                             void* stream);
 
 /*
  * The kernels of the reference's point-to-point microbenchmarks as HIP kernels

@@ -15,11 +15,18 @@ is.
 
 import os as _os
 
-from . import _native
-from .iris import Iris, iris
-from .util import do_bench, memset_tensor
+# One process per rank: peers map each other's heaps through hipIpcOpenMemHandle, and on hosts whose driver
+# only supports dmabuf IPC that needs HSA_ENABLE_IPC_MODE_LEGACY=0 in the environment before the HIP runtime
+# initialises (else hipIpcGetMemHandle fails with "invalid argument").  A value the user set is kept.
+_os.environ.setdefault("HSA_ENABLE_IPC_MODE_LEGACY", "0")
 
-__all__ = ["Iris", "iris", "do_bench", "memset_tensor", "use_finegrained_allocator"]
+from . import _native  # noqa: E402
+from ._bootstrap import launched_as_ranks  # noqa: E402
+from .iris import IPC_MAX_HEAP_BYTES, Iris, iris  # noqa: E402
+from .util import do_bench, memset_tensor  # noqa: E402
+
+__all__ = ["Iris", "iris", "do_bench", "memset_tensor", "use_finegrained_allocator", "launched_as_ranks",
+           "IPC_MAX_HEAP_BYTES"]
 
 
 def use_finegrained_allocator():

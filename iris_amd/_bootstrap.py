@@ -60,9 +60,13 @@ class StoreComm:
         if self.rank == root:
             assert value is not None, "Root must provide a value."
             arr = np.array(value)
-            self.store.set(key, arr.dtype.str.encode() + b"|" + arr.tobytes())
-        dtype, _, raw = bytes(self.store.get(key)).partition(b"|")
-        return np.frombuffer(raw, dtype=np.dtype(dtype.decode()))[0]
+            # one length byte, the dtype's name, the value's bytes (a one-byte dtype's name itself starts with
+            # '|': "|b1", "|i1", "|u1", so no separator character is safe)
+            name = arr.dtype.str.encode()
+            self.store.set(key, bytes([len(name)]) + name + arr.tobytes())
+        blob = bytes(self.store.get(key))
+        n = blob[0]
+        return np.frombuffer(blob[1 + n:], dtype=np.dtype(blob[1:1 + n].decode()))[0]
 
     def barrier(self):
         self._exchange(b"\x01")
@@ -97,6 +101,16 @@ class MpiComm:
 
 def _under_mpi_launcher() -> bool:
     return any(k in os.environ for k in ("OMPI_COMM_WORLD_SIZE", "PMI_SIZE", "PMIX_RANK", "MV2_COMM_WORLD_SIZE"))
+
+
+def launched_as_ranks() -> bool:
+    """Whether this process was started as one rank of several (what
+    ``init_comm`` would find), without opening a store or initialising MPI."""
+    if int(os.environ.get("WORLD_SIZE", "1")) > 1:
+        return True
+    if os.environ.get("IRIS_AMD_RENDEZVOUS") is None and _under_mpi_launcher():
+        return importlib.util.find_spec("mpi4py") is not None
+    return False
 
 
 def init_comm():

@@ -14,6 +14,8 @@ import threading
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libiris_amd.so")
 ALLOCATOR_LIB_PATH = os.path.join(_PKG_DIR, "csrc", "finegrained_alloc", "libfinegrained_allocator.so")
+# kernels that only the tests and bench.py call (include/iris_amd_testing.h)
+TESTING_LIB_PATH = os.path.join(_PKG_DIR, "libiris_amd_testing.so")
 
 # element types (IRIS_DTYPE_*)
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
@@ -27,6 +29,8 @@ SCOPE_AGENT, SCOPE_SYSTEM = 0, 1
 VARIANT_FEW_ROWS, VARIANT_PERSISTENT = 1000, 1001
 SPLIT_STREAM_K = -1  # GemmArgs.split_k: stream-K
 HANDOVER_AUTO, HANDOVER_OWNER, HANDOVER_SLICED = 0, 1, 2  # GemmArgs.split_handover
+# how a tile's flag orders its data (IRIS_FLAG_SEM_*)
+FLAG_SEM_WRITE_THROUGH, FLAG_SEM_RELEASE_ACQUIRE = 0, 1
 # status word (IRIS_STATUS_*)
 STATUS_OK, STATUS_SPIN_TIMEOUT = 0, 1
 
@@ -79,6 +83,7 @@ class GemmArgs(ctypes.Structure):
         ("partials_slot_elems", ctypes.c_int64),
         ("split_k", ctypes.c_int32),
         ("split_handover", ctypes.c_int32),
+        ("flag_sem", ctypes.c_int32),
     ]
 
 
@@ -110,6 +115,7 @@ class ReduceArgs(ctypes.Structure):
         ("wait_flags", ctypes.c_int32),
         ("variant", ctypes.c_int32),
         ("spin_timeout_ticks", ctypes.c_uint64),
+        ("flag_sem", ctypes.c_int32),
     ]
 
 
@@ -145,16 +151,20 @@ SIGNATURES = {
     "iris_tile_map_host": (None, [ctypes.c_int32] * 6 + [ctypes.POINTER(ctypes.c_int32)] * 2),
     "iris_stream_k_schedule_host": (_I, [ctypes.c_int32] * 4 + [ctypes.POINTER(ctypes.c_int32), ctypes.c_int32,
                                          ctypes.POINTER(ctypes.c_int32)]),
-    "iris_mfma_probe_launch": (_I, [_P, _P, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P]),
-    "iris_store_probe_launch": (_I, [_P, _P, _P, ctypes.c_uint64] + [ctypes.c_int32] * 5 + [_P]),
-    "iris_rma_selftest_launch": (_I, [ctypes.c_int32] * 4 + [_P, _P, _P] + [ctypes.c_int32] * 3 + [_P]),
     "iris_p2p_bench_launch": (_I, [ctypes.c_int32] * 2 + [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 3
                               + [_P, ctypes.c_int32, _P]),
     "iris_amd_abi_version": (_I, []),
 }
 ALLOCATOR_SYMBOLS = ("finegrained_hipMalloc", "finegrained_hipFree")
+# every symbol include/iris_amd_testing.h declares for libiris_amd_testing.so
+TESTING_SIGNATURES = {
+    "iris_mfma_probe_launch": (_I, [_P, _P, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P]),
+    "iris_store_probe_launch": (_I, [_P, _P, _P, ctypes.c_uint64] + [ctypes.c_int32] * 5 + [_P]),
+    "iris_rma_selftest_launch": (_I, [ctypes.c_int32] * 4 + [_P, _P, _P] + [ctypes.c_int32] * 3 + [_P]),
+}
 
 _lib = None
+_testing_lib = None
 _lock = threading.Lock()
 
 
@@ -177,6 +187,24 @@ def lib() -> ctypes.CDLL:
                 fn.argtypes = argtypes
             _lib = handle
     return _lib
+
+
+def testing_lib() -> ctypes.CDLL:
+    """Load ``libiris_amd_testing.so`` (tests and bench.py only) once and type its entry points."""
+    global _testing_lib
+    if _testing_lib is not None:
+        return _testing_lib
+    with _lock:
+        if _testing_lib is None:
+            if not os.path.exists(TESTING_LIB_PATH):
+                raise RuntimeError(f"{TESTING_LIB_PATH} not found. Build it with `python -m iris_amd.build`.")
+            handle = ctypes.CDLL(TESTING_LIB_PATH)
+            for name, (restype, argtypes) in TESTING_SIGNATURES.items():
+                fn = getattr(handle, name)
+                fn.restype = restype
+                fn.argtypes = argtypes
+            _testing_lib = handle
+    return _testing_lib
 
 
 def hip_try(err: int) -> None:

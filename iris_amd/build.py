@@ -1,4 +1,4 @@
-"""Build the two shared libraries of the package with hipcc for gfx950.
+"""Build the shared libraries of the package with hipcc for gfx950.
 
     python -m iris_amd.build            # build what is out of date
     python -m iris_amd.build --force    # rebuild everything
@@ -7,6 +7,9 @@
 this file, ``libfinegrained_allocator.so`` to ``csrc/finegrained_alloc/`` --
 the place the reference's package looks for it (iris/__init__.py:29-38; built
 there by setup.py:22-84 / csrc/finegrained_alloc/build.sh).
+``libiris_amd_testing.so`` (``csrc/testing/``: measurement probes and unit-test
+kernels that only the tests and bench.py call) is a library of its own, so
+that the product library exports nothing but the product's entry points.
 """
 
 from __future__ import annotations
@@ -24,6 +27,7 @@ CSRC = PKG / "csrc"
 OBJ = CSRC / "build"
 LIB = PKG / "libiris_amd.so"
 ALLOC_LIB = CSRC / "finegrained_alloc" / "libfinegrained_allocator.so"
+TESTING_LIB = PKG / "libiris_amd_testing.so"
 
 ARCH = "gfx950"
 # packed-fp32 instructions are kept out of all device code
@@ -49,8 +53,13 @@ def kernel_sources():
     return sorted(p for p in CSRC.glob("*.hip"))
 
 
+def testing_sources():
+    return sorted(p for p in (CSRC / "testing").glob("*.hip"))
+
+
 def _headers():
-    return list(CSRC.glob("*.hpp")) + [PKG.parent / "include" / "iris_amd.h"]
+    inc = PKG.parent / "include"
+    return list(CSRC.glob("*.hpp")) + [inc / "iris_amd.h", inc / "iris_amd_testing.h", inc / "iris_device.hpp"]
 
 
 def _stale(target: Path, deps) -> bool:
@@ -74,12 +83,13 @@ def build(force: bool = False, jobs: int | None = None, verbose: bool = True) ->
     jobs = jobs or min(8, os.cpu_count() or 1)
 
     todo = []
-    objs = []
-    for src in kernel_sources():
-        obj = OBJ / (src.stem + ".o")
-        objs.append(obj)
-        if force or _stale(obj, [src] + hdrs):
-            todo.append((src, obj))
+    objs, testing_objs = [], []
+    for sources, into in ((kernel_sources(), objs), (testing_sources(), testing_objs)):
+        for src in sources:
+            obj = OBJ / (src.stem + ".o")
+            into.append(obj)
+            if force or _stale(obj, [src] + hdrs):
+                todo.append((src, obj))
 
     def compile_one(item):
         src, obj = item
@@ -95,6 +105,10 @@ def build(force: bool = False, jobs: int | None = None, verbose: bool = True) ->
         _run([cc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)])
         if verbose:
             print(f"[iris_amd.build] linked {LIB.name}", flush=True)
+    if force or todo or _stale(TESTING_LIB, testing_objs):
+        _run([cc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(TESTING_LIB), *map(str, testing_objs)])
+        if verbose:
+            print(f"[iris_amd.build] linked {TESTING_LIB.name}", flush=True)
 
     alloc_src = CSRC / "finegrained_alloc" / "finegrained_allocator.hip"
     if force or _stale(ALLOC_LIB, [alloc_src]):

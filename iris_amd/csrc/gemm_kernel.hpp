@@ -46,6 +46,8 @@
 
 namespace iris_amd {
 
+constexpr int FLAG_MODE_MASK = 3, FLAG_RELEASE = 4;
+
 struct GemmKArgs {
   const char* a;
   const char* b;
@@ -70,7 +72,9 @@ struct GemmKArgs {
   FastDiv div_subs, div_sub_n;  // sub_m * sub_n, sub_n
   FastDiv div_split, div_nk;    // split_k; K-steps of a tile (stream-K runs)
   int dest_all;      // write `out` on every rank's heap (else on this rank only)
-  int flag_mode;     // 0: none, 1: +1 on every rank, 2: +1 on every other rank
+  // bits 1:0 -- 0: none, 1: +1 on every rank, 2: +1 on every other rank;  bit 2 (FLAG_RELEASE): the +1 is a
+  // release at the flags' scope, as the reference's sem="release" (else relaxed, behind write-through stores)
+  int flag_mode;
   int sys;           // flag atomics at system scope (else agent)
   int vec_out;       // 16-byte vector access allowed on `out`
   // > 0 (split-K launches with long parts; the value is total_tiles): the programs are numbered part by part
@@ -713,6 +717,8 @@ __device__ __attribute__((always_inline)) inline bool store_acc(const GemmKArgs&
 // tile to complete and the group has passed a barrier.  Those stores were
 // write-through at the flag's scope, so they are already visible there and
 // the increment itself can be relaxed: it is ordered after them by the waits.
+// (This has been validated with producers and consumers on ONE device only; a
+// launch may ask for the reference's release instead, FLAG_RELEASE.)
 // Lane l takes ranks l, l + 64, ...: the ranks' heap bases come in with one
 // vector load and the increments leave together (one thread walking the ranks
 // waits for a scalar load per rank: 0.8 us for eight).
@@ -735,11 +741,14 @@ __device__ __attribute__((always_inline)) inline void publish_tile(const GemmKAr
       if constexpr (merged) first = tile_id_of(pm0 + i, pn0 + j, p.flag_num_pid_m, p.flag_num_pid_n, p.G);
       IRIS_GLOBAL int32_t* own = (IRIS_GLOBAL int32_t*)(p.flags + first);
       for (int r = lane; r < p.ws; r += 64) {
-        if (p.flag_mode == 2 && r == p.cur_rank) continue;
+        if ((p.flag_mode & FLAG_MODE_MASK) == 2 && r == p.cur_rank) continue;
         IRIS_GLOBAL int32_t* f = own;
         if (r != p.cur_rank && p.heap_bases != nullptr)
           f = translate(p.flags + first, p.heap_bases[p.cur_rank], p.heap_bases[r]);
-        flag_add_relaxed(f, 1, p.sys != 0);
+        if (p.flag_mode & FLAG_RELEASE)
+          flag_add_release(f, 1, p.sys != 0);  // gemm_one_shot_all_reduce.py:207-218 verbatim
+        else
+          flag_add_relaxed(f, 1, p.sys != 0);
       }
     }
 }
@@ -1496,6 +1505,10 @@ gemm_persistent_kernel(const GemmKArgs p) {
   if (n_items > 0) c_it = decode_item<Cfg, SPLIT>(p, sr, pid, 0);
 
   // end of a compute tile: store it, and publish the logical tile it completes
+  // FUSED: a wait for a peer's tile has timed out.  The peer is not resident (or gone): the tiles that follow
+  // are still stored and signalled, but not waited for, so that a launch without its peers costs one timeout
+  // and not one per tile.
+  int peers_gone = 0;
   auto epilogue = [&]() __attribute__((always_inline)) {
     if (defer_publish && pending_tile >= 0) {
       // a one-step tile: the previous tile has not been published yet
@@ -1600,13 +1613,14 @@ gemm_persistent_kernel(const GemmKArgs p) {
         if (p.ws > 1) {
           if (wave == 0) publish_tile<MERGED>(p, c_it.tile_id, lane);  // +1 on every other rank (:207-218)
           if (tid == 0) {
-            *slot = wait_tile_flag((IRIS_GLOBAL int32_t*)(p.flags + c_it.tile_id), p.ws, p.sys != 0, p.timeout,
-                                   p.status)
+            *slot = !peers_gone && wait_tile_flag((IRIS_GLOBAL int32_t*)(p.flags + c_it.tile_id), p.ws, p.sys != 0,
+                                                  p.timeout, p.status)
                         ? 1
                         : 0;  // CAS(ws-1 -> 0) until it succeeds (:220-234), bounded
           }
           __syncthreads();
           ok = *slot;
+          if (!ok) peers_gone = 1;
         }
         if (ok) {
           // rows in flight per lane (the accumulators' registers are free by now)

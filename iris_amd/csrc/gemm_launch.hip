@@ -393,8 +393,11 @@ hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan) {
       return hipErrorInvalidValue;
   }
   if (out_dt != IRIS_DTYPE_F32 && out_dt != a.ab_dtype) return hipErrorInvalidValue;
+  if (a.flag_sem != IRIS_FLAG_SEM_WRITE_THROUGH && a.flag_sem != IRIS_FLAG_SEM_RELEASE_ACQUIRE)
+    return hipErrorInvalidValue;
+  if (k.flag_mode != 0 && a.flag_sem == IRIS_FLAG_SEM_RELEASE_ACQUIRE) k.flag_mode |= FLAG_RELEASE;
   if (k.flag_mode != 0 && a.world_size > 1 && !a.tile_completed) return hipErrorInvalidValue;
-  if (k.flag_mode == 1 && !a.tile_completed) return hipErrorInvalidValue;
+  if ((k.flag_mode & FLAG_MODE_MASK) == 1 && !a.tile_completed) return hipErrorInvalidValue;
   if (a.M == 0 || a.N == 0) return hipSuccess;  // nothing to compute
   if (!a.a || !a.b) {
     if (a.K > 0) return hipErrorInvalidValue;
@@ -573,6 +576,7 @@ iris_reduce_args reduce_args_from(const iris_gemm_args& a) {
   r.wait_flags = 1;
   r.variant = 0;
   r.spin_timeout_ticks = a.spin_timeout_ticks;
+  r.flag_sem = a.flag_sem;
   return r;
 }
 

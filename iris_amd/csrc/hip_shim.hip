@@ -73,6 +73,6 @@ int iris_hip_arch_name(int device, char* buf, size_t len) {
   return hipSuccess;
 }
 
-int iris_amd_abi_version(void) { return 4; }
+int iris_amd_abi_version(void) { return 5; }
 
 }  // extern "C"

@@ -34,6 +34,9 @@ struct ReduceKArgs {
   // row-band kernel: the group that finishes last takes the consumed flags
   // back to 0 (else the launcher enqueues reset_consumed_flags_kernel)
   int reset_in_kernel;
+  // an acquire fence at the flags' scope after every flag wait, as the reference's sem="acquire" (the loads are
+  // coherent at that scope by themselves and need none)
+  int acquire;
 };
 
 // The row-band kernel counts its finished groups in the upper half of the
@@ -50,7 +53,7 @@ __device__ inline bool block_wait_tile(const ReduceKArgs& p, int tile_id, IRIS_L
     *slot = wait_tile_flag((IRIS_GLOBAL int32_t*)(p.flags + tile_id), p.ws, p.sys != 0, p.timeout, p.status) ? 1 : 0;
   __syncthreads();
   const int ok = *slot;
-  if constexpr (FENCE) {
+  if (FENCE || p.acquire) {
     if (p.sys)
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
     else
@@ -220,6 +223,12 @@ __global__ __launch_bounds__(256) void reduce_rows_kernel(const ReduceKArgs p) {
         ready[tid] = ok;
       }
       all = __syncthreads_and(ok) != 0;
+      if (p.acquire) {
+        if (p.sys)
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+        else
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      }
     }
     uint32_t ioff[K], ooff[K];
 #pragma unroll

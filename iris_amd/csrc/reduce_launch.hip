@@ -100,6 +100,9 @@ extern "C" int iris_one_shot_reduce_launch(const iris_reduce_args* a, void* stre
   k.cg_dt = a->c_global_dtype;
   k.sys = a->scope == IRIS_SCOPE_SYSTEM;
   k.wait_flags = a->wait_flags;
+  if (a->flag_sem != IRIS_FLAG_SEM_WRITE_THROUGH && a->flag_sem != IRIS_FLAG_SEM_RELEASE_ACQUIRE)
+    return hipErrorInvalidValue;
+  k.acquire = a->flag_sem == IRIS_FLAG_SEM_RELEASE_ACQUIRE;
 
   // default grid: two blocks per CU, each walking its share of the tiles
   int grid = a->num_sms > 0 ? a->num_sms : 2 * current_cu_count();

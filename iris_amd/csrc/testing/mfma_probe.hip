@@ -7,7 +7,8 @@
 // peak, is what a GEMM kernel on the same data can approach.
 #include <hip/hip_runtime.h>
 
-#include "common.hpp"
+#include "../../../include/iris_amd_testing.h"
+#include "../common.hpp"
 
 namespace iris_amd {
 

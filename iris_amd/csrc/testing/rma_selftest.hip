@@ -5,8 +5,8 @@
 // target in turn.  C-ABI: iris_rma_selftest_launch.
 #include <hip/hip_runtime.h>
 
-#include "../../include/iris_amd.h"
-#include "../../include/iris_device.hpp"
+#include "../../../include/iris_amd_testing.h"
+#include "../../../include/iris_device.hpp"
 
 namespace {
 

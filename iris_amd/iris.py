@@ -77,6 +77,8 @@ def _finegrained_pool(nbytes: int, device: str) -> torch.Tensor:
 
 # hipIpcOpenMemHandle has been seen not to return for larger allocations
 _IPC_MAX_BYTES = (2 << 30) - 1
+# the largest heap a launcher should default to with one process per rank: 2 GiB less one allocation unit
+IPC_MAX_HEAP_BYTES = (2 << 30) - (1 << 20)
 
 
 class Iris:

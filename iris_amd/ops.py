@@ -32,6 +32,8 @@ from ._native import (
     HANDOVER_AUTO,
     HANDOVER_OWNER,
     HANDOVER_SLICED,
+    FLAG_SEM_WRITE_THROUGH,
+    FLAG_SEM_RELEASE_ACQUIRE,
 )
 
 __all__ = [
@@ -41,7 +43,6 @@ __all__ = [
     "gemm_plan_name",
     "stream_k_schedule_host",
     "gemm_variant_name",
-    "store_probe",
     "one_shot_reduce",
     "signal_tiles",
     "tile_schedule",
@@ -57,6 +58,8 @@ __all__ = [
     "PHASE_TWO_KERNELS",
     "SCOPE_AGENT",
     "SCOPE_SYSTEM",
+    "FLAG_SEM_WRITE_THROUGH",
+    "FLAG_SEM_RELEASE_ACQUIRE",
 ]
 
 _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
@@ -64,11 +67,7 @@ _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: D
 # limits of iris_gemm_launch_noalloc (include/iris_amd.h)
 NOALLOC_MAX_PROGRAMS, NOALLOC_MAX_TILE_ELEMS = 256, 16384
 
-# iris_rma_selftest_launch (include/iris_amd.h)
-RMA_OPS = {"load": 0, "store": 1, "get": 2, "put": 3, "atomic_add": 4, "atomic_sub": 5, "atomic_cas": 6,
-           "atomic_xchg": 7}
-RMA_SEMS = {"relaxed": 0, "acquire": 1, "release": 2, "acq_rel": 3}
-RMA_SCOPES = {"cta": 2, "gpu": SCOPE_AGENT, "sys": SCOPE_SYSTEM}
+# element types of iris_p2p_bench_launch beside the floating-point ones (include/iris_amd.h)
 _RMA_DTYPES = dict(_DTYPES)
 _RMA_DTYPES.update({torch.int8: 3, torch.int16: 4, torch.int32: 5, torch.int64: 6})
 
@@ -233,8 +232,14 @@ def _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_s
 def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
                 gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, scope=SCOPE_AGENT, variant=0,
                 mm_begin_timestamp=None, mm_end_timestamp=None, status=None, spin_timeout_ticks=0, partials=None,
-                locks=None, split_k=0, noalloc=False, split_handover=HANDOVER_AUTO):
+                locks=None, split_k=0, noalloc=False, split_handover=HANDOVER_AUTO,
+                flag_sem=FLAG_SEM_WRITE_THROUGH):
     """Launch the persistent shard GEMM ``a @ b`` with a tile-publishing epilogue.
+
+    ``flag_sem``: ``FLAG_SEM_WRITE_THROUGH`` (write-through stores, then a
+    relaxed flag add: validated with concurrent producers and consumers on one
+    device) or ``FLAG_SEM_RELEASE_ACQUIRE`` (the reference's
+    ``sem="release"`` on the flag add, gemm_one_shot_all_reduce.py:207-218).
 
     ``partials`` / ``locks`` are the wrappers' ``P`` and ``locks`` buffers
     (matmul_wrapper.py:29-31): with them, a launch with far fewer tiles than
@@ -271,6 +276,7 @@ def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size,
                                split_k)
         launch = _native.lib().iris_gemm_launch
     args.split_handover = split_handover
+    args.flag_sem = flag_sem
     stream = torch.cuda.current_stream(a.device).cuda_stream
     with torch.cuda.device(a.device):
         err = launch(ctypes.byref(args), stream)
@@ -347,11 +353,14 @@ def stream_k_schedule_host(total_tiles: int, k_steps: int, num_programs: int, pi
 
 def one_shot_reduce(c, c_global, tile_completed, heap_bases, rank, world_size, BLK_M, BLK_N, gsize_m, *,
                     num_sms=0, num_xcds=1, scope=SCOPE_AGENT, wait_flags=True, variant=0, status=None,
-                    spin_timeout_ticks=0):
+                    spin_timeout_ticks=0, flag_sem=FLAG_SEM_WRITE_THROUGH):
     """Sum the ``world_size`` partial buffers that sit at ``c``'s heap offset on
     every rank into ``c_global``, tile by tile, behind the tiles' flags.
 
     The consumer half of gemm_one_shot_all_reduce.py:220-271.
+    ``flag_sem=FLAG_SEM_RELEASE_ACQUIRE`` adds the reference's acquire after
+    every flag wait (:220-234); by default the loads are coherent at the
+    flags' scope by themselves.
     """
     if c.dim() != 2 or c_global.dim() != 2:
         raise ValueError("c and c_global must be matrices")
@@ -384,6 +393,7 @@ def one_shot_reduce(c, c_global, tile_completed, heap_bases, rank, world_size, B
     args.wait_flags = 1 if wait_flags else 0
     args.variant = variant
     args.spin_timeout_ticks = spin_timeout_ticks
+    args.flag_sem = flag_sem
     stream = torch.cuda.current_stream(device).cuda_stream
     with torch.cuda.device(device):
         err = _native.lib().iris_one_shot_reduce_launch(ctypes.byref(args), stream)
@@ -412,62 +422,6 @@ def tile_map_host(tile_id, M, N, BLK_M, BLK_N, gsize_m):
     pm, pn = ctypes.c_int32(), ctypes.c_int32()
     _native.lib().iris_tile_map_host(tile_id, M, N, BLK_M, BLK_N, gsize_m, ctypes.byref(pm), ctypes.byref(pn))
     return pm.value, pn.value
-
-
-def mfma_probe(operands, sink, iters, num_groups):
-    """Launch the register-only MFMA loop (a measurement aid): returns the FLOP
-    count of the launch.  ``operands``: >= 64 KiB of fp16/bf16 on the device,
-    ``sink``: >= num_groups * 512 floats."""
-    if operands.dtype not in _DTYPES or operands.dtype == torch.float32:
-        raise ValueError("operands must be fp16 or bf16")
-    if operands.numel() * operands.element_size() < 65536 or sink.numel() < num_groups * 512:
-        raise ValueError("operands: at least 64 KiB; sink: at least num_groups * 512 floats")
-    if sink.dtype != torch.float32 or not operands.is_contiguous():
-        raise ValueError("sink must be fp32 and operands contiguous")
-    stream = torch.cuda.current_stream(operands.device).cuda_stream
-    _native.hip_try(_native.lib().iris_mfma_probe_launch(_ptr(operands), _ptr(sink), _DTYPES[operands.dtype], iters,
-                                                         num_groups, ctypes.c_void_p(stream)))
-    return num_groups * 8 * iters * 16 * 16384
-
-
-def store_probe(operands, sink, out, tiles, chunk, num_groups, *, write_through=True, lockstep=True):
-    """Launch the store probe (a measurement aid): ``tiles`` tiles per group of
-    8 waves, each 16 K-steps of register-only MFMAs and 128 KiB of stores to
-    ``out``, ``chunk`` one-KiB stores a wave back to back every ``chunk``
-    K-steps (16, 4, 1, or 0 for none).  Returns the bytes stored per launch."""
-    if operands.dtype != torch.bfloat16 or operands.numel() * 2 < 65536 or not operands.is_contiguous():
-        raise ValueError("operands: at least 64 KiB of contiguous bf16")
-    if sink.dtype != torch.float32 or sink.numel() < num_groups * 512:
-        raise ValueError("sink: at least num_groups * 512 floats")
-    out_bytes = out.numel() * out.element_size()
-    if not out.is_contiguous() or out_bytes < num_groups * 131072:
-        raise ValueError("out: contiguous, at least 128 KiB per group")
-    stream = torch.cuda.current_stream(operands.device).cuda_stream
-    err = _native.lib().iris_store_probe_launch(_ptr(operands), _ptr(sink), _ptr(out), out_bytes, tiles, chunk,
-                                                1 if write_through else 0, 1 if lockstep else 0, num_groups,
-                                                ctypes.c_void_p(stream))
-    if err == _native.HIP_ERROR_INVALID_VALUE:
-        raise ValueError("iris_store_probe_launch rejected the arguments")
-    _native.hip_try(err)
-    return 0 if chunk == 0 else tiles * num_groups * 131072
-
-
-def rma_selftest(op, data, results, heap_bases, rank, num_ranks, block_size, *, sem="acq_rel", scope="sys"):
-    """Run one of the unit-test kernels over the device-side remote-access
-    functions (include/iris_device.hpp) as rank ``rank``: ``op`` is a key of
-    ``RMA_OPS``, ``sem`` / ``scope`` the reference's strings
-    (tests/unittests/test_atomic_add.py:44-60)."""
-    if results.dtype not in _RMA_DTYPES:
-        raise ValueError(f"unsupported element type {results.dtype}")
-    if data is not None and data.dtype != results.dtype:
-        raise ValueError("data and results must have the same element type")
-    if not 1 <= block_size <= 64 or results.numel() < block_size or (data is not None and data.numel() < block_size):
-        raise ValueError("block_size must be 1..64 and fit the buffers")
-    _check_heap_bases(heap_bases, num_ranks, results.device)
-    stream = torch.cuda.current_stream(results.device).cuda_stream
-    _native.hip_try(_native.lib().iris_rma_selftest_launch(
-        RMA_OPS[op], _RMA_DTYPES[results.dtype], RMA_SEMS[sem], RMA_SCOPES[scope], _ptr(data), _ptr(results),
-        _ptr(heap_bases), rank, num_ranks, block_size, ctypes.c_void_p(stream)))
 
 
 # iris_p2p_bench_launch (include/iris_amd.h)

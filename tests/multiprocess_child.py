@@ -19,7 +19,7 @@ sys.path.insert(0, ROOT)
 import torch  # noqa: E402
 
 import iris_amd  # noqa: E402
-from iris_amd import ops  # noqa: E402
+from iris_amd import ops, testing  # noqa: E402
 from oracle import iris_oracle as O  # noqa: E402
 
 
@@ -56,22 +56,22 @@ def main():
         for block in (1, 8, 32):
             for op, expect in (("load", ws), ("store", 1), ("get", ws), ("put", 1)):
                 data, results = fresh(block, dtype, 1, 0)
-                ops.rma_selftest(op, data, results, hb, rank, ws, block)
+                testing.rma_selftest(op, data, results, hb, rank, ws, block)
                 check(results, expect, f"{op} {dtype} block {block}")
     for dtype in (torch.int32, torch.int64, torch.float16, torch.bfloat16, torch.float32):
         for sem, scope in (("relaxed", "gpu"), ("release", "sys"), ("acq_rel", "sys"), ("acquire", "gpu")):
             _, results = fresh(16, dtype, 1, 0)
-            ops.rma_selftest("atomic_add", None, results, hb, rank, ws, 16, sem=sem, scope=scope)
+            testing.rma_selftest("atomic_add", None, results, hb, rank, ws, 16, sem=sem, scope=scope)
             check(results, ws, f"atomic_add {dtype} {sem} {scope}")
     _, results = fresh(16, torch.int32, 1, 2 * ws)
-    ops.rma_selftest("atomic_sub", None, results, hb, rank, ws, 16)
+    testing.rma_selftest("atomic_sub", None, results, hb, rank, ws, 16)
     check(results, ws, "atomic_sub")
     for dtype in (torch.int32, torch.int64):
         _, results = fresh(1, dtype, 1, 0)
-        ops.rma_selftest("atomic_cas", None, results, hb, rank, ws, 1, sem="acq_rel", scope="sys")
+        testing.rma_selftest("atomic_cas", None, results, hb, rank, ws, 1, sem="acq_rel", scope="sys")
         check(results, ws, f"atomic_cas {dtype}")
         _, results = fresh(1, dtype, 1, 0)
-        ops.rma_selftest("atomic_xchg", None, results, hb, rank, ws, 1, sem="acq_rel", scope="sys")
+        testing.rma_selftest("atomic_xchg", None, results, hb, rank, ws, 1, sem="acq_rel", scope="sys")
         check(results, ws, f"atomic_xchg {dtype}")
     say("remote-access kernels ok")
 

@@ -1,5 +1,6 @@
-"""The C-ABI: both libraries load and export every symbol ``include/iris_amd.h``
-declares, and the ctypes structs have the layout the C compiler gives them.
+"""The C-ABI: the libraries load and export every symbol ``include/iris_amd.h``
+(the product) and ``include/iris_amd_testing.h`` (test and bench kernels)
+declare, and the ctypes structs have the layout the C compiler gives them.
 No compute call is made."""
 
 import ctypes
@@ -14,10 +15,11 @@ from iris_amd import _native
 
 ROOT = os.path.abspath(os.path.join(os.path.dirname(__file__), ".."))
 HEADER = os.path.join(ROOT, "include", "iris_amd.h")
+TESTING_HEADER = os.path.join(ROOT, "include", "iris_amd_testing.h")
 
 
-def declared_functions():
-    text = open(HEADER).read()
+def declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(iris_[a-z0-9_]+|finegrained_hip[A-Za-z]+)\s*\(", text)))
 
@@ -27,13 +29,23 @@ def test_header_and_bindings_name_the_same_functions():
     lib_names = [n for n in names if n.startswith("iris_")]
     assert sorted(lib_names) == sorted(_native.SIGNATURES)
     assert sorted(n for n in names if n.startswith("finegrained_")) == sorted(_native.ALLOCATOR_SYMBOLS)
+    assert declared_functions(TESTING_HEADER) == sorted(_native.TESTING_SIGNATURES)
+
+
+def test_the_product_library_exports_no_test_or_probe_kernel():
+    lib = ctypes.CDLL(_native.LIB_PATH)
+    for name in _native.TESTING_SIGNATURES:
+        assert not hasattr(lib, name), f"{name} belongs to libiris_amd_testing.so"
 
 
 def test_libraries_load_and_export_every_declared_symbol():
     lib = _native.lib()
     for name in _native.SIGNATURES:
         assert getattr(lib, name) is not None
-    assert lib.iris_amd_abi_version() == 4
+    assert lib.iris_amd_abi_version() == 5
+    testing = _native.testing_lib()
+    for name in _native.TESTING_SIGNATURES:
+        assert getattr(testing, name) is not None
     alloc = ctypes.CDLL(_native.ALLOCATOR_LIB_PATH)
     for name in _native.ALLOCATOR_SYMBOLS:
         assert getattr(alloc, name) is not None

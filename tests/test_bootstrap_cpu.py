@@ -32,6 +32,10 @@ v = comm.broadcast_scalar(3.5 + r if r == 1 else None, root=1)
 assert float(v) == 4.5
 n = comm.broadcast_scalar(np.int64(41 + r) if r == 0 else None, root=0)
 assert int(n) == 41
+# one-byte element types (their dtype names start with '|')
+assert bool(comm.broadcast_scalar(True if r == 0 else None, root=0)) is True
+assert int(comm.broadcast_scalar(np.int8(-7) if r == 0 else None, root=0)) == -7
+assert int(comm.broadcast_scalar(np.uint8(200) if r == 1 else None, root=1)) == 200
 for _ in range(5):
     comm.barrier()
 print("RANK", r, "OK")

@@ -16,6 +16,7 @@ import torch
 from iris_amd import ops
 from oracle import iris_oracle as O
 
+from parity import default_scale
 from test_gemm_gpu import check_close, make_ab, to_heap
 
 pytestmark = pytest.mark.gpu
@@ -62,12 +63,20 @@ def two_streams(shmem_gpu):
     pytest.fail("no two streams of this process run side by side on the device")
 
 
+# Concurrent passes per parametrisation, each on fresh operands.  Every wait is bounded and every kernel exits;
+# the loop stops at the first mismatch or timeout.
+ROUNDS = 50
+
+
+@pytest.mark.parametrize("flag_sem", [ops.FLAG_SEM_WRITE_THROUGH, ops.FLAG_SEM_RELEASE_ACQUIRE])
 @pytest.mark.parametrize("scope", [ops.SCOPE_AGENT, ops.SCOPE_SYSTEM])
 @pytest.mark.parametrize("variant", [7, 8])  # row bands, tiles
 @pytest.mark.parametrize("ws", [2, 4])
-def test_one_shot_consumer_polls_while_producers_publish(shmem, two_streams, ws, variant, scope):
+def test_one_shot_consumer_polls_while_producers_publish(shmem, two_streams, ws, variant, scope, flag_sem):
     """09 split in two kernels: ranks 1..ws-1 produce (partial tile stores +
-    flag +1 on rank 0) while rank 0's consumer is already waiting."""
+    flag +1 on rank 0) while rank 0's consumer is already waiting.  With the
+    default flag semantics (write-through stores, relaxed flag) and with the
+    reference's release / acquire."""
     M = N = 4096
     K, BM, BN, G = 2048, 128, 128, 6
     dtype = torch.bfloat16
@@ -80,57 +89,71 @@ def test_one_shot_consumer_polls_while_producers_publish(shmem, two_streams, ws,
     status = torch.zeros(1, dtype=torch.int32, device="cuda")
     hb = shmem.get_heap_bases()
     on = shmem.on_rank
-    for r in range(ws):
-        for t in (c, cg, flags):
-            on(t, r).zero_()
+    scale = float(A.float().std())
+
+    def clear():
+        for r in range(ws):
+            for t in (c, cg, flags):
+                on(t, r).zero_()
 
     def produce(r, grid):
         ops.gemm_launch(a_full[:, r * K:(r + 1) * K], b_full[r * K:(r + 1) * K, :], on(c, r), on(cg, r),
                         on(flags, r), hb, r, ws, grid, BM, BN, 64, G, ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE,
-                        num_xcds=8, scope=scope, status=status)
+                        num_xcds=8, scope=scope, status=status, flag_sem=flag_sem)
 
     def consume():
         ops.one_shot_reduce(c, cg, flags, hb, 0, ws, BM, BN, G, num_sms=128, num_xcds=8, scope=scope,
-                            variant=variant, status=status, spin_timeout_ticks=HALF_SECOND)
+                            variant=variant, status=status, spin_timeout_ticks=HALF_SECOND, flag_sem=flag_sem)
 
-    # one pass in stream order first: every kernel is loaded and its result known
-    for r in range(ws):
-        produce(r, 128)
-    consume()
-    torch.cuda.synchronize()
-    want = cg.cpu()
-    assert int(status.item()) == 0 and flags.cpu().tolist() == [0] * total
-    for r in range(ws):
-        for t in (c, cg, flags):
-            on(t, r).zero_()
-
-    # rank 0's own partial is stream-ordered before its consumer, as in the reference program
-    produce(0, 256)
-    torch.cuda.synchronize()
     sa, sb = two_streams
-    cons_begin, cons_end, prod_end = (torch.cuda.Event(enable_timing=True) for _ in range(3))
-    # the consumer goes first: its 128 blocks leave at least 128 CUs empty for the producers' 128 programs
-    with torch.cuda.stream(sb):
-        cons_begin.record()
-        consume()
-        cons_end.record()
-    with torch.cuda.stream(sa):
-        for r in range(1, ws):
+    zeros = torch.zeros(total, dtype=torch.int32, device="cuda")
+    others = torch.full((total,), ws - 1, dtype=torch.int32, device="cuda")
+    leads = []
+    for it in range(ROUNDS):
+        if it > 0:  # fresh operands, drawn on the device
+            a_full.normal_(0, scale)
+        # one pass in stream order first: the result of these operands is known (and every kernel is loaded)
+        clear()
+        for r in range(ws):
             produce(r, 128)
-        prod_end.record()
-    torch.cuda.synchronize()
-    assert int(status.item()) == 0, "a flag wait timed out: the kernels did not overlap as planned"
-    # the consumer was on the device before the producers were done, and cannot have finished before them
-    lead, lag = cons_begin.elapsed_time(prod_end), prod_end.elapsed_time(cons_end)
-    print(f"consumer enqueued {lead * 1e3:.0f} us before the producers finished, done {lag * 1e3:.0f} us after them")
-    assert lead > 0, "the consumer started after the producers had finished: nothing was polled"
-    assert torch.equal(cg.cpu(), want), "the concurrent pass differs from the pass in stream order"
-    partials = torch.stack([on(c, r).cpu() for r in range(ws)])
-    assert torch.equal(cg.cpu(), O.one_shot_reduce(partials, dtype)), "consumer read a partial before it was complete"
-    assert flags.cpu().tolist() == [0] * total
-    for r in range(1, ws):  # the other ranks' flags: +1 from everyone but themselves, never consumed
-        assert on(flags, r).cpu().tolist() == [ws - 1] * total
-    check_close(cg, O.one_shot_all_reduce(O.k_shards(A, B, ws), torch.float32, dtype), "vs closed form")
+        consume()
+        torch.cuda.synchronize()
+        want = cg.clone()
+        assert int(status.item()) == 0 and torch.equal(flags, zeros), f"round {it}, stream order"
+        # A consumer that reads a partial before it is complete must find something else there: zeros
+        clear()
+        # rank 0's own partial is stream-ordered before its consumer, as in the reference program
+        produce(0, 256)
+        torch.cuda.synchronize()
+        cons_begin, cons_end, prod_end = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        # the consumer goes first: its 128 blocks leave at least 128 CUs empty for the producers' 128 programs
+        with torch.cuda.stream(sb):
+            cons_begin.record()
+            consume()
+            cons_end.record()
+        with torch.cuda.stream(sa):
+            for r in range(1, ws):
+                produce(r, 128)
+            prod_end.record()
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0, f"round {it}: a flag wait timed out: the kernels did not overlap as planned"
+        # the consumer was on the device before the producers were done, and cannot have finished before them
+        lead, lag = cons_begin.elapsed_time(prod_end), prod_end.elapsed_time(cons_end)
+        leads.append((lead, lag))
+        assert lead > 0, f"round {it}: the consumer started after the producers had finished: nothing was polled"
+        assert torch.equal(cg, want), f"round {it}: the concurrent pass differs from the pass in stream order"
+        assert torch.equal(flags, zeros), f"round {it}: flags not consumed"
+        for r in range(1, ws):  # the other ranks' flags: +1 from everyone but themselves, never consumed
+            assert torch.equal(on(flags, r), others), f"round {it}: flags of rank {r}"
+        if it in (0, ROUNDS - 1):
+            # against the oracle: the rank-ordered sum of the partials, bit for bit, and the closed form
+            partials = torch.stack([on(c, r).cpu() for r in range(ws)])
+            assert torch.equal(cg.cpu(), O.one_shot_reduce(partials, dtype)), "not the rank-ordered sum"
+            Ah, Bh = a_full.cpu(), b_full.cpu()
+            check_close(cg, O.one_shot_all_reduce(O.k_shards(Ah, Bh, ws), torch.float32, dtype), "vs closed form")
+    lead, lag = leads[-1]
+    print(f"{ROUNDS} rounds; last: consumer enqueued {lead * 1e3:.0f} us before the producers finished, "
+          f"done {lag * 1e3:.0f} us after them")
 
 
 @pytest.mark.parametrize("scope", [ops.SCOPE_AGENT, ops.SCOPE_SYSTEM])
@@ -189,6 +212,7 @@ def test_scatter_ready_flags_gate_a_concurrent_reader(shmem, two_streams, scope)
     assert flags.cpu().tolist() == [0] * total and on(flags, 1).cpu().tolist() == [1] * total
 
 
+@pytest.mark.parametrize("flag_sem", [ops.FLAG_SEM_WRITE_THROUGH, ops.FLAG_SEM_RELEASE_ACQUIRE])
 @pytest.mark.parametrize("scope", [ops.SCOPE_AGENT, ops.SCOPE_SYSTEM])
 @pytest.mark.parametrize("M,N,K,BM,BN,partial_dtype", [
     (4096, 4096, 512, 256, 256, torch.float32),   # 256 tiles, two per program, one compute tile each
@@ -199,15 +223,19 @@ def test_scatter_ready_flags_gate_a_concurrent_reader(shmem, two_streams, scope)
     (300, 250, 136, 128, 64, torch.float32),      # N no multiple of four: the element-wise reduce
 ])
 def test_one_shot_inside_the_program_two_ranks_side_by_side(shmem, two_streams, M, N, K, BM, BN, partial_dtype,
-                                                            scope):
+                                                            scope, flag_sem):
     """IRIS_PHASE_FUSED, the reference program's own order
     (gemm_one_shot_all_reduce.py:197-271): each program stores its partial
     tile, signals the other rank, waits for the tile's flag on its own rank,
     sums the tile over both ranks and stores it, tile by tile.  Two ranks of
-    128 programs each share the 256 CUs, one stream per rank."""
+    128 programs each share the 256 CUs, one stream per rank.  ROUNDS passes,
+    each on fresh operands."""
     ws, G = 2, 6
     dtype = torch.bfloat16
-    A, B = make_ab(M, N, K * ws, dtype, seed=M + N)
+    # 16-bit partials round at 2^-9 of their own size, which can be more than the tolerance allows the (smaller)
+    # sum when two large partials cancel: those cases keep their partials well below 1
+    shrink = 0.3 if partial_dtype != torch.float32 else 1.0
+    A, B = make_ab(M, N, K * ws, dtype, seed=M + N, scale=shrink * default_scale(K * ws))
     a_full, b_full = to_heap(shmem, A), to_heap(shmem, B)
     c = shmem.zeros((M, N), dtype=partial_dtype)
     cg = shmem.zeros((M, N), dtype=dtype)
@@ -225,20 +253,30 @@ def test_one_shot_inside_the_program_two_ranks_side_by_side(shmem, two_streams, 
                 ws, 128, BM, BN, 64, G, ops.EPI_ONE_SHOT)
         kw = dict(phase=ops.PHASE_FUSED, num_xcds=8)
         assert ops.gemm_plan_name(*args, **kw).endswith("+reduce")
-        ops.gemm_launch(*args, status=status, spin_timeout_ticks=HALF_SECOND, scope=scope, **kw)
+        ops.gemm_launch(*args, status=status, spin_timeout_ticks=HALF_SECOND, scope=scope, flag_sem=flag_sem, **kw)
 
-    torch.cuda.synchronize()
-    for r, s in enumerate(two_streams):
-        with torch.cuda.stream(s):
-            launch(r)
-    torch.cuda.synchronize()
-    assert int(status.item()) == 0, "a program gave up waiting for its peer"
-    partials = torch.stack([on(c, r).cpu() for r in range(ws)])
-    shards = O.k_shards(A, B, ws)
-    for r in range(ws):
-        check_close(partials[r], O.shard_gemm(*shards[r], partial_dtype), f"partial of rank {r}")
-    want = O.one_shot_reduce(partials, dtype)
-    for r in range(ws):
-        assert torch.equal(on(cg, r).cpu(), want), f"rank {r}: not the rank-ordered sum of the partials"
-        assert on(flags, r).cpu().tolist() == [0] * total  # every flag went up once and was consumed
-    check_close(cg, O.one_shot_all_reduce(shards, partial_dtype, dtype), "vs closed form")
+    scale = float(A.float().std())
+    zeros = torch.zeros(total, dtype=torch.int32, device="cuda")
+    for it in range(ROUNDS):
+        if it > 0:  # fresh operands, drawn on the device; the partials of the round before are still in `c`
+            a_full.normal_(0, scale)
+        torch.cuda.synchronize()
+        for r, s in enumerate(two_streams):
+            with torch.cuda.stream(s):
+                launch(r)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0, f"round {it}: a program gave up waiting for its peer"
+        # two ranks: the rank-ordered fp32 sum is one addition, which the device computes to the same bits
+        want_dev = (on(c, 0).float() + on(c, 1).float()).to(dtype)
+        for r in range(ws):
+            assert torch.equal(on(cg, r), want_dev), f"round {it}, rank {r}: not the sum of the partials"
+            assert torch.equal(on(flags, r), zeros), f"round {it}, rank {r}: flags"  # up once, consumed
+        if it in (0, ROUNDS - 1):
+            partials = torch.stack([on(c, r).cpu() for r in range(ws)])
+            shards = O.k_shards(a_full.cpu(), b_full.cpu(), ws)
+            for r in range(ws):
+                check_close(partials[r], O.shard_gemm(*shards[r], partial_dtype), f"partial of rank {r}")
+            want = O.one_shot_reduce(partials, dtype)
+            for r in range(ws):
+                assert torch.equal(on(cg, r).cpu(), want), f"rank {r}: not the rank-ordered sum of the partials"
+            check_close(cg, O.one_shot_all_reduce(shards, partial_dtype, dtype), "vs closed form")

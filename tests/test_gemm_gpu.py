@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from iris_amd import ops
+from iris_amd import ops, testing
 from oracle import iris_oracle as O
 from parity import ATOL, RTOL, blocks_ok, check_close, make_ab  # noqa: F401  (re-exported to the other GPU test modules)
 
@@ -423,7 +423,7 @@ def test_store_probe_writes_every_groups_region(shmem):
     for chunk in (16, 4, 1):
         for wt in (True, False):
             out = torch.full((tiles * groups * 131072 + 4096,), 0x5A, dtype=torch.uint8, device="cuda")
-            assert ops.store_probe(operands, sink, out[:-4096], tiles, chunk, groups, write_through=wt) == tiles * groups * 131072
+            assert testing.store_probe(operands, sink, out[:-4096], tiles, chunk, groups, write_through=wt) == tiles * groups * 131072
             torch.cuda.synchronize()
             body = out[:-4096].view(torch.float32)
             # accumulators of ones x ones products: whole numbers, never the fill pattern
@@ -431,13 +431,13 @@ def test_store_probe_writes_every_groups_region(shmem):
             assert not bool((out[:-4096] == 0x5A).view(-1, 16).all(dim=1).any()), "a 16-byte unit was not written"
             assert bool((out[-4096:] == 0x5A).all())
     out = torch.full((groups * 131072,), 0x5A, dtype=torch.uint8, device="cuda")
-    assert ops.store_probe(operands, sink, out, tiles, 0, groups) == 0
+    assert testing.store_probe(operands, sink, out, tiles, 0, groups) == 0
     torch.cuda.synchronize()
     assert bool((out == 0x5A).all()) and bool(torch.isfinite(sink).all())
     with pytest.raises(ValueError):
-        ops.store_probe(operands, sink, out[:1000], tiles, 16, groups)
+        testing.store_probe(operands, sink, out[:1000], tiles, 16, groups)
     with pytest.raises(ValueError):
-        ops.store_probe(operands, sink, out, tiles, 3, groups)
+        testing.store_probe(operands, sink, out, tiles, 3, groups)
 
 
 def _fetching_wave_cases():

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import iris_amd
-from iris_amd import ops
+from iris_amd import ops, testing
 
 pytestmark = pytest.mark.gpu
 
@@ -41,7 +41,7 @@ def run_all_ranks(heap, op, data, results, block, **kw):
     n = heap.get_num_ranks()
     hb = heap.get_heap_bases()
     for r in range(n):
-        ops.rma_selftest(op, None if data is None else heap.on_rank(data, r), heap.on_rank(results, r), hb, r, n, block,
+        testing.rma_selftest(op, None if data is None else heap.on_rank(data, r), heap.on_rank(results, r), hb, r, n, block,
                          **kw)
     torch.cuda.synchronize()
 
@@ -151,6 +151,6 @@ def test_cas_only_swaps_on_a_match_and_masked_lanes_do_nothing(heap):
 def test_selftest_launcher_rejects_bad_arguments(heap):
     _, results = fresh(heap, 8, torch.int8, 1)
     with pytest.raises(RuntimeError):  # int8 has no atomics
-        ops.rma_selftest("atomic_add", None, results, heap.get_heap_bases(), 0, heap.get_num_ranks(), 8)
+        testing.rma_selftest("atomic_add", None, results, heap.get_heap_bases(), 0, heap.get_num_ranks(), 8)
     with pytest.raises(ValueError):
-        ops.rma_selftest("load", results, results, heap.get_heap_bases(), 0, heap.get_num_ranks(), 65)
+        testing.rma_selftest("load", results, results, heap.get_heap_bases(), 0, heap.get_num_ranks(), 65)

@@ -36,6 +36,34 @@ def run_pair(shmem, M, N, K, BM, BN, grid, dtype, split_k, expect_split):
     assert f_na.cpu().tolist() == f_ws.cpu().tolist() == [1] * total
 
 
+def test_noalloc_allocates_nothing(shmem):
+    """The property the entry point exists for: once the first call on the
+    device has looked the library's array up, a call leaves the device's free
+    memory and torch's allocator exactly as it found them."""
+    dtype = torch.bfloat16
+    A, B = make_ab(100, 200, 1024, dtype, seed=3)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((100, 200), dtype=dtype)
+    flags = shmem.zeros((8,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+
+    def call():
+        ops.gemm_launch(a, b, None, cg, flags, hb, 0, 1, 256, 64, 64, 64, 2, ops.EPI_ALL_SCATTER, split_k=8,
+                        noalloc=True)
+
+    call()  # (the symbol lookup, and the kernels' code objects loaded)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    held0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, f"device memory in use changed by {free0 - free1} bytes"
+    assert torch.cuda.memory_allocated() == held0 and torch.cuda.memory_reserved() == reserved0
+    check_close(cg, O.shard_gemm(A, B, dtype))
+
+
 def test_noalloc_matches_the_workspace_launch_twice(shmem):
     # split-K 8 on 64 x 64 tiles, then a smaller input with another split
     run_pair(shmem, 100, 200, 1024, 64, 64, 256, torch.bfloat16, 8, 8)
@@ -109,6 +137,19 @@ def test_noalloc_limits_are_errors(shmem):
     assert _native.lib().iris_gemm_launch_noalloc(ctypes.byref(args), None) == _native.HIP_ERROR_INVALID_VALUE
     args.num_sms, args.block_m, args.block_n, args.split_k = 256, 256, 256, 2
     assert _native.lib().iris_gemm_launch_noalloc(ctypes.byref(args), None) == _native.HIP_ERROR_INVALID_VALUE
+    # stream-K forced on a tile larger than a slot: rejected like any forced split, in the wrapper and in the library
+    with pytest.raises(ValueError, match="forced split"):
+        ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 16, 256, 128, 64, 2, ops.EPI_ALL_SCATTER,
+                        split_k=ops.SPLIT_STREAM_K, noalloc=True)
+    args.num_sms, args.block_m, args.block_n, args.split_k = 16, 256, 128, ops.SPLIT_STREAM_K
+    assert _native.lib().iris_gemm_launch_noalloc(ctypes.byref(args), None) == _native.HIP_ERROR_INVALID_VALUE
+    # exactly as many programs as the array has slots is inside the limit
+    cg64, f64 = shmem.zeros((256, 256), dtype=dtype), shmem.zeros((16,), dtype=torch.int32)
+    ops.gemm_launch(a, b, None, cg64, f64, None, 0, 1, ops.NOALLOC_MAX_PROGRAMS, 64, 64, 64, 2, ops.EPI_ALL_SCATTER,
+                    split_k=8, noalloc=True)
+    torch.cuda.synchronize()
+    check_close(cg64, O.shard_gemm(A, B, dtype), "256 programs, split 8")
+    assert f64.cpu().tolist() == [1] * 16
     # without a forced split a large tile simply runs unsplit
     ops.gemm_launch(a, b, None, cg, flags, None, 0, 1, 256, 256, 256, 64, 2, ops.EPI_ALL_SCATTER, noalloc=True)
     torch.cuda.synchronize()
