@@ -8,10 +8,14 @@ the bf16 shard GEMM A[8192,1024] x B[1024,8192] (one rank's K-shard of
 K=8192) with 256x256 output tiles stored as bf16 into the fine-grained heap
 and one uint32 ready flag published per tile.  Prints ONE JSON line.
 
-Also measured and reported inside that line: the one-shot reduce of 8 fp32
-partial-C buffers [8192,8192] -> bf16 (the reduce phase, HBM-bound), the same
-GEMM under the reference's cold-cache ``do_bench`` protocol, and a CPU
-baseline of the same math on the host cores.
+The last line printed is the result: the GEMM's figures, and inside its
+``roofline`` object also the reduce phase (``roofline.reduce``: the one-shot
+reduce of 8 fp32 partial-C buffers [8192,8192] -> bf16, HBM-bound), the CPU
+baseline of the same math on the host cores, and one-line summaries of the
+other measurements.  Everything else (the cold-cache protocol run, the
+library and matrix-core context figures, the other workloads) is printed
+before it, one JSON line per group, each with a ``detail`` key, so that the
+result line stays short.
 """
 
 import argparse
@@ -70,11 +74,13 @@ def parse():
     ap.add_argument("--shapes-gpus", default="1,2,4,8", help="shapes workload: the GPU counts the GEMMs are cut over")
     ap.add_argument("--shapes-algorithms", default="all_scatter,one_shot",
                     help="shapes workload: all_scatter (N-shards) and / or one_shot (K-shards, the producer)")
-    ap.add_argument("--workload", choices=["headline", "atomic", "decoder", "shapes"], default="headline",
+    ap.add_argument("--workload", choices=["headline", "atomic", "decoder", "shapes", "fused"], default="headline",
                     help="headline: the 8192x8192x1024 shard GEMM + reduce (the metric's configuration); atomic: eight "
                          "K-shard GEMMs adding into one fp32 C; decoder: 6.7B-decoder-shaped shards for M in "
                          "{1,16,128,512,2048}; shapes: one rank's shard GEMM at every point of the reference's shape "
-                         "sweep, beside the vendor library's.  The last three print their own JSON line.")
+                         "sweep, beside the vendor library's; fused: the reference's one-shot program (store, signal, "
+                         "wait, reduce, tile by tile) on two ranks resident side by side, against the producer + "
+                         "reduce-kernel pair.  The last four print their own JSON line.")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="headline run: skip the atomic-accumulate and decoder-shard summaries")
     ap.add_argument("--no-context", action="store_true",
@@ -320,6 +326,197 @@ def run_atomic(args, emit=True):
     if emit:
         print(json.dumps(result))
     return result
+
+
+def side_by_side_streams(shmem):
+    """Two streams of this process that really run side by side on the device.
+    HIP maps streams onto a few hardware queues and two streams on one queue run
+    one after the other, so candidate pairs are probed with the flag protocol
+    itself: a one-tile consumer with a bounded wait (20 ms) on one stream, then
+    the signal it waits for on the other."""
+    import torch
+
+    from iris_amd import ops
+
+    off = shmem.heap_offset
+    ws = shmem.get_num_ranks()
+    c = shmem.zeros((64, 64), dtype=torch.float32)
+    cg = shmem.zeros((64, 64), dtype=torch.float32)
+    flag = shmem.zeros((1,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    for st in streams:  # the first submission to a new stream takes milliseconds
+        with torch.cuda.stream(st):
+            torch.zeros(8, device="cuda").add_(1)
+    torch.cuda.synchronize()
+    try:
+        for sb in streams:
+            for sa in streams:
+                if sa is sb:
+                    continue
+                for r in range(ws):
+                    shmem.on_rank(flag, r).zero_()
+                status.zero_()
+                torch.cuda.synchronize()
+                with torch.cuda.stream(sb):
+                    ops.one_shot_reduce(c, cg, flag, hb, 0, 2, 64, 64, 1, num_sms=1, variant=8, status=status,
+                                        spin_timeout_ticks=2_000_000)
+                with torch.cuda.stream(sa):
+                    ops.signal_tiles(shmem.on_rank(flag, 1), hb, 1, 1, 2)
+                torch.cuda.synchronize()
+                if int(status.item()) == 0:
+                    return sa, sb
+    finally:
+        shmem.heap_offset = off
+    raise RuntimeError("no two streams of this process run side by side on the device")
+
+
+def run_fused(args, emit=True):
+    """The reference's 09 program as it runs (gemm_one_shot_all_reduce.py:197-271):
+    every program stores its partial tile, signals the other rank, waits for
+    the tile's flag on its own rank, sums the tile over the ranks and stores
+    it, tile by tile.  Two ranks of 128 programs each, resident side by side
+    on the one GPU (one stream per rank), each computing
+    [8192, 1024] x [1024, 8192] of a K = 2048 product into fp32 partials and a
+    bf16 result; against the same work as two kernels per rank on one stream
+    (producer GEMM on 256 programs, then the reduce kernel)."""
+    import torch
+
+    import iris_amd
+    from iris_amd import ops
+    from oracle import iris_oracle as O
+
+    ws, ks = 2, K_SHARD
+    blk_m, blk_n, gsize = 256, 256, 6  # the 09 script's own tile and group size
+    half_second = 50_000_000            # every wait is bounded: 0.5 s of the 100 MHz wall clock
+    shmem = iris_amd.iris(1 << 30, virtual_ranks=ws)
+    on = shmem.on_rank
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(123)
+    A = (torch.randn(M, ks * ws, generator=g) * 0.02).to(dtype)
+    B = (torch.randn(N, ks * ws, generator=g) * 0.02).to(dtype)
+    a_full = shmem.zeros((M, ks * ws), dtype=dtype)
+    a_full.copy_(A)
+    bt_full = shmem.zeros((N, ks * ws), dtype=dtype)
+    bt_full.copy_(B)
+    del A, B
+    c = shmem.zeros((M, N), dtype=torch.float32)
+    cg = shmem.zeros((M, N), dtype=dtype)
+    total = ops.cdiv(M, blk_m) * ops.cdiv(N, blk_n)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    hb = shmem.get_heap_bases()
+    xcds = ops.default_num_xcds(shmem.get_cu_count(), 128)
+    sa, sb = side_by_side_streams(shmem)
+
+    def clear():
+        for r in range(ws):
+            for t in (c, cg, flags):
+                on(t, r).zero_()
+        status.zero_()
+
+    def launch(r, phase, grid):
+        ops.gemm_launch(a_full[:, r * ks:(r + 1) * ks], bt_full[:, r * ks:(r + 1) * ks].T, on(c, r), on(cg, r),
+                        on(flags, r), hb, r, ws, grid, blk_m, blk_n, 64, gsize, ops.EPI_ONE_SHOT, phase=phase,
+                        num_xcds=xcds, status=status, spin_timeout_ticks=half_second)
+
+    def in_program():  # both ranks' programs on the device together
+        for r, st in enumerate((sa, sb)):
+            with torch.cuda.stream(st):
+                launch(r, ops.PHASE_FUSED, 128)
+
+    def two_kernels():  # both producers, then both reduce kernels, on one stream
+        for r in range(ws):
+            launch(r, ops.PHASE_PRODUCE, 256)
+        for r in range(ws):
+            ops.one_shot_reduce(on(c, r), on(cg, r), on(flags, r), hb, r, ws, blk_m, blk_n, gsize, num_xcds=xcds,
+                                status=status, spin_timeout_ticks=half_second)
+
+    # correctness first, on the whole matrices: the partials against each other's builds, and the result of both
+    # forms bit for bit against the oracle's rank-ordered sum of those partials
+    results = {}
+    for name, run in (("in_program", in_program), ("two_kernels", two_kernels)):
+        clear()
+        torch.cuda.synchronize()
+        run()
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0, f"{name}: a flag wait timed out"
+        partials = torch.stack([on(c, r).cpu() for r in range(ws)])
+        want = O.one_shot_reduce(partials, dtype)
+        for r in range(ws):
+            assert torch.equal(on(cg, r).cpu(), want), f"{name}: rank {r} is not the rank-ordered sum of the partials"
+            assert int(on(flags, r).abs().max().item()) == 0, f"{name}: flags of rank {r} not consumed"
+        results[name] = partials
+    assert torch.equal(results["in_program"], results["two_kernels"]), "the two forms computed different partials"
+    del results, partials, want
+
+    steps = max(5, min(args.steps, 100))
+    start, end_a, end_b = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+
+    def timed_in_program():
+        ms = []
+        for _ in range(steps):
+            torch.cuda.synchronize()
+            with torch.cuda.stream(sa):
+                start.record()
+            sb.wait_event(start)
+            in_program()
+            with torch.cuda.stream(sa):
+                end_a.record()
+            with torch.cuda.stream(sb):
+                end_b.record()
+            torch.cuda.synchronize()
+            ms.append(max(start.elapsed_time(end_a), start.elapsed_time(end_b)))
+        return ms
+
+    def timed_two_kernels():
+        ms = []
+        for _ in range(steps):
+            torch.cuda.synchronize()
+            start.record()
+            two_kernels()
+            end_a.record()
+            torch.cuda.synchronize()
+            ms.append(start.elapsed_time(end_a))
+        return ms
+
+    # settle the clocks on this work, then alternate the two forms
+    t_end = time.perf_counter() + args.settle_ms * 1e-3
+    while time.perf_counter() < t_end:
+        two_kernels()
+        torch.cuda.synchronize()
+    timed_in_program()
+    t_in, t_two = timed_in_program(), timed_two_kernels()
+    assert int(status.item()) == 0, "a flag wait timed out during the timed runs"
+    for r in range(ws):
+        assert int(on(flags, r).abs().max().item()) == 0
+    ms_in, ms_two = statistics.median(t_in), statistics.median(t_two)
+    flops = ws * 2.0 * M * N * ks
+    rbytes = ws * (ws * M * N * 4 + M * N * 2)
+    out = {
+        "metric": "one-shot all-reduce GEMM as the reference program runs it (store, signal, wait, reduce per tile), "
+                  "two ranks side by side on one GPU",
+        "value": round(flops / (ms_in * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps,
+        "ms_per_step": round(ms_in, 5), "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "2 ranks x 128 programs of IRIS_PHASE_FUSED, each [8192,1024] x [1024,8192] (K-shard views "
+                               "of K = 2048), 256x256 tiles, fp32 partials, bf16 result on both ranks; one stream per rank",
+                   "ranks": ws, "programs_per_rank": 128, "BLK_M": blk_m, "BLK_N": blk_n, "gsize_m": gsize},
+        "in_program": {"ms": round(ms_in, 5), "min_ms": round(min(t_in), 5), "max_ms": round(max(t_in), 5),
+                       "tflops": round(flops / (ms_in * 1e-3) / 1e12, 2)},
+        "two_kernels": {"what": "the same work as kernels on one stream: both ranks' producer GEMMs (256 programs), then "
+                                "both ranks' reduce kernels", "ms": round(ms_two, 5), "min_ms": round(min(t_two), 5),
+                        "max_ms": round(max(t_two), 5), "tflops": round(flops / (ms_two * 1e-3) / 1e12, 2)},
+        "in_program_vs_two_kernels": round(ms_two / ms_in, 3),
+        "reduce_bytes": rbytes,
+        "checked": "both forms bit-exact against the oracle's rank-ordered sum of the partials on the whole "
+                   "[8192,8192], flags back to 0, status 0",
+    }
+    if emit:
+        print(json.dumps(out))
+    del shmem
+    return out
+
 
 
 # The reference's shape sweep (examples/benchmark/bench_all_shapes.py:103-187): the six GEMMs of
@@ -647,6 +844,8 @@ def main():
         return run_decoder(args)
     if args.workload == "shapes":
         return run_shapes(args)
+    if args.workload == "fused":
+        return run_fused(args)
 
     ws = 8
     # per-rank heap: full-K operands 2 x 128 MiB, bf16 results 2 x 128 MiB, fp32 partial 256 MiB, flags
@@ -699,6 +898,7 @@ def main():
     regs, spills = ops.gemm_kernel_info(a, b, None, c_global, flags, hb, 0, 1, GRID, BLK_M, BLK_N, BLK_K,
                                         args.gsize_m, ops.EPI_ALL_SCATTER, num_xcds=num_xcds, variant=args.variant)
 
+    details = {}  # printed before the result line, one JSON line per entry
     result = {
         "metric": "fused GEMM+reduce TFLOP/s (% bf16 MFMA peak); reduce-phase HBM GB/s",
         "value": round(tflops, 2),
@@ -741,9 +941,7 @@ def main():
         cold_tflops = flops / (cold_ms * 1e-3) / 1e12
         result["gemm_cold_cache"] = {"protocol": "do_bench: 256 MiB cache flush before every repetition, mean of 50",
                                      "ms": round(cold_ms, 5), "tflops": round(cold_tflops, 2),
-                                     "roofline": {"bound": "mfma", "achieved": round(cold_tflops, 2),
-                                                  "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                                                  "frac": round(cold_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}}
+                                     "frac": round(cold_tflops / PEAK_BF16_TFLOPS, 4)}
         if not args.no_context:
             # the vendor library's GEMM on the same operands under the same protocol (no flags)
             lib_out = torch.empty((M, N), dtype=dtype, device="cuda")
@@ -792,14 +990,16 @@ def main():
         rbytes = ws * M * N * 4 + M * N * 2
         rms = statistics.mean(red_ms)
         gbps = rbytes / (rms * 1e-3) / 1e9
-        result["reduce"] = {
+        # the reduce half of the metric, inside `roofline` so that it travels with the GEMM's
+        result["roofline"]["reduce"] = {
             "workload": "one-shot reduce of 8 fp32 partial-C [8192,8192] -> bf16, gated by per-tile flags",
-            "mean_ms": round(rms, 5), "launches": steps, "GBps": round(gbps, 1),
-            "pct_of_hbm_peak": round(100.0 * gbps / PEAK_HBM_GBPS, 2), "variant": args.reduce_variant,
-            "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                         "frac": round(gbps / PEAK_HBM_GBPS, 4),
-                         "traffic": REDUCE_TRAFFIC_BYTES if args.reduce_variant == 0 else None},
+            "bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+            "frac": round(gbps / PEAK_HBM_GBPS, 4),
+            "traffic": REDUCE_TRAFFIC_BYTES if args.reduce_variant == 0 else None,
+            "ms": round(rms, 5), "launches": steps, "variant": args.reduce_variant,
         }
+        result["reduce_GBps"] = round(gbps, 1)
+        result["pct_of_hbm_peak"] = round(100.0 * gbps / PEAK_HBM_GBPS, 2)
         if not args.no_context:
             # the same launch with other numbers of groups (the default is two per CU): the rate follows the
             # groups a CU hosts, not the bytes it requests; 10 launches each, flags armed beforehand as above
@@ -819,12 +1019,22 @@ def main():
                 e.record()
                 torch.cuda.synchronize()
                 sweep[str(groups)] = round(rbytes / (s.elapsed_time(e) / 10 * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
-            result["reduce"]["frac_by_groups"] = sweep
+            details["reduce_frac_by_groups"] = sweep
 
     if not args.no_context:
         # (after the two headline measurements: seconds of probes at the power cap in front of the reduce's
         # thirty launches would be measured with them)
-        result["context"] = context_figures(a, b, c_global, flops, gemm_on)
+        ctx = context_figures(a, b, c_global, flops, gemm_on)
+        details["context"] = ctx
+        # the one-line version for the result line: the vendor library's plain GEMM on the same operands, this
+        # kernel and the library on zeros, what the matrix cores alone sustain on such data
+        result["context"] = {
+            "library_gemm_ms": ctx["library_gemm"]["ms"],
+            "gemm_on_zeros_ms": ctx["gemm_on_zeros"]["ms"],
+            "library_gemm_on_zeros_ms": ctx["library_gemm_on_zeros"]["ms"],
+            "mfma_only_tflops_on_such_data": ctx["mfma_sustained[random N(0,0.02)]"]["tflops"],
+            "mfma_only_tflops_on_zeros": ctx["mfma_sustained[zeros]"]["tflops"],
+        }
 
     if args.copy_calibration:
         # ws=1, fp32 -> fp32: the reduce kernel degenerates to a plain tiled copy
@@ -847,7 +1057,8 @@ def main():
                 "library_gate_up_us", "library_down_us", "at_reference_default_tile_256x64")
         args.shapes_gpus = "8"  # (the whole sweep, 1 to 8 GPUs, is the --workload shapes run)
         sweep = run_shapes(args, emit=False)
-        result["other_workloads"] = {
+        fz = run_fused(args, emit=False)
+        details["other_workloads"] = {
             "atomic_accumulate": {k: at[k] for k in ("value", "unit", "ms_per_step", "atomic_updates_per_s",
                                                      "atomic_ceiling", "config")},
             "decoder_shards": {"config": dec["config"], "per_M": [{k: r[k] for k in keep} for r in dec["per_M"]]},
@@ -856,11 +1067,30 @@ def main():
                                    "points": [{k: pt[k] for k in ("algorithm", "shard", "tile", "kernel", "split_k",
                                                                   "us", "tflops", "library_us", "vs_library")}
                                               for pt in sweep["points"]]},
+            "one_shot_in_program": {k: fz[k] for k in ("config", "in_program", "two_kernels",
+                                                       "in_program_vs_two_kernels", "checked")},
+        }
+        # one line each for the result line
+        result["other_workloads"] = {
+            "atomic_accumulate_ms": at["ms_per_step"],
+            "atomic_frac_of_atomic_ceiling": at["atomic_ceiling"]["frac_of_ceiling"],
+            "decoder_gate_up_us_by_M": {str(r["M"]): r["gate_up_us"] for r in dec["per_M"]},
+            "decoder_library_gate_up_us_by_M": {str(r["M"]): r["library_gate_up_us"] for r in dec["per_M"]},
+            "decoder_down_us_by_M": {str(r["M"]): r["down_us"] for r in dec["per_M"]},
+            "decoder_library_down_us_by_M": {str(r["M"]): r["library_down_us"] for r in dec["per_M"]},
+            "shape_sweep_8_gpus_vs_library": {"geomean": sweep["value"], "worst": sweep["worst"],
+                                              "best": sweep["best"]},
+            "one_shot_in_program_2_ranks_ms": fz["in_program"]["ms"],
+            "one_shot_two_kernels_2_ranks_ms": fz["two_kernels"]["ms"],
         }
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
 
+    # the groups of detail first, one line each; the result line last
+    for name, value in details.items():
+        print(json.dumps({"detail": name, name: value}))
+    sys.stdout.flush()
     print(json.dumps(result))
 
 
