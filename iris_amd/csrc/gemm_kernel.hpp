@@ -138,26 +138,12 @@ struct Mfma<IRIS_DTYPE_BF16> {
   __device__ static inline f32x4 run(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
-  // the same with the accumulator pinned to the accumulation registers (tiles of 256 accumulators a lane:
-  // they fill that half of the register file exactly, and the fragments keep the other half)
-  __device__ static inline void run_acc(vec8 a, vec8 b, f32x4& c) {
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-  }
-  __device__ static inline void first_acc(vec8 a, vec8 b, f32x4& c) {
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
-  }
 };
 template <>
 struct Mfma<IRIS_DTYPE_F16> {
   using vec8 = f16x8;
   __device__ static inline f32x4 run(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
-  }
-  __device__ static inline void run_acc(vec8 a, vec8 b, f32x4& c) {
-    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-  }
-  __device__ static inline void first_acc(vec8 a, vec8 b, f32x4& c) {
-    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
   }
 };
 
@@ -172,9 +158,7 @@ struct GemmCfg {
   static constexpr int DT = DT_, CM = CM_, CN = CN_, BK = BK_, WM = WM_, WN = WN_, S = S_;
   static constexpr bool DMA = DMA_;
   static constexpr int NW = WM * WN, NT = NW * 64;  // the waves (threads) that multiply and store
-  // LW_ == 1 marks the four-wave 256 x 256 tile whose stages are refilled by LDS-DMA (no wave only fetches)
-  static constexpr bool BIG_DMA = LW_ == 1;
-  static constexpr int LW = BIG_DMA ? 0 : LW_;
+  static constexpr int LW = LW_;
   static constexpr int NL = LW ? LW : NW;           // the waves that fetch
   static constexpr int THREADS = (NW + LW) * 64;    // launch size
   static constexpr int TM = CM / WM, TN = CN / WN;
@@ -196,7 +180,7 @@ struct GemmCfg {
   static constexpr bool SPLITK = DMA_ && KSUB % 2 == 0 && IM * IN * 4 <= 128;
   static constexpr bool SPLIT_OWNER = SPLITK && IM * IN * 4 <= 64;
   // Waves per SIMD the register budget is sized for: 256 registers a wave.
-  static constexpr int WPE = IM * IN * 4 > 128 ? 1 : 2;
+  static constexpr int WPE = 2;
   // wave-private epilogue scratch: 32 rows x TN 16-bit elements
   static constexpr int WS_PITCH = TN * 2;
   static constexpr int WS_BYTES = 32 * WS_PITCH;
@@ -212,8 +196,7 @@ struct GemmCfg {
   static_assert(S >= 1, "ring depth");
   static_assert(!DMA || S >= 2, "the DMA ring needs a stage being read and one in flight");
   static_assert(L * (S - 1) <= 63, "vmcnt immediate");
-  static_assert(IM * IN * 4 <= 256, "accumulators of a wave tile: at most 256 registers");
-  static_assert(IM * IN * 4 <= 128 || NW + LW <= 4, "256 accumulators a lane: one wave per SIMD");
+  static_assert(IM * IN * 4 <= 128, "accumulators of a wave tile: at most 128 registers (two waves a SIMD)");
   static_assert(TN == 32 || TN == 64 || TN == 128, "wave tile width");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
@@ -496,12 +479,7 @@ template <class Cfg, bool FIRST>
 __device__ inline void mma_row(f32x4 (&acc)[Cfg::IM][Cfg::IN], const Frags<Cfg>& f, int cb, int i) {
 #pragma unroll
   for (int j = 0; j < Cfg::IN; ++j) {
-    if constexpr (Cfg::IM * Cfg::IN * 4 > 128) {
-      if constexpr (FIRST)
-        Mfma<Cfg::DT>::first_acc(f.b[cb][j], f.a[i], acc[i][j]);
-      else
-        Mfma<Cfg::DT>::run_acc(f.b[cb][j], f.a[i], acc[i][j]);
-    } else if constexpr (FIRST) {
+    if constexpr (FIRST) {
       const f32x4 z = {0, 0, 0, 0};
       acc[i][j] = Mfma<Cfg::DT>::run(f.b[cb][j], f.a[i], z);
     } else {
@@ -1056,355 +1034,6 @@ __device__ inline void fused_reduce_tile(const GemmKArgs& p, const Item& it, int
 // The kernel
 // ---------------------------------------------------------------------------
 
-// The K loop of the tiles whose wave holds 256 accumulators a lane (256 x 256 as 2 x 2 waves of 128 x 128): one
-// wave per SIMD with the whole register file, the accumulators in its accumulation half.  A 128 x 128 wave tile
-// reads 16 fragments from LDS for 64 MFMAs where the 128 x 64 one reads 12 for 32, and with that the K loop is
-// bound by the matrix cores instead of by LDS.  Stages are 32 deep in a ring of four: step g multiplies the
-// fragments it fetched during step g-1, fetches those of step g+1 from the stage that landed last, and refills
-// the stage it just left with step g+4, one load per block of MFMAs.  Unsplit, one compute tile per logical
-// tile; the flag of a tile is published once the tile's stores have completed.
-//
-// A tuning variant, not the launcher's choice: with one wave per SIMD every load the wave issues holds its
-// MFMAs up, and no fetching wave fits beside a wave of 512 registers.  [8192,7168] x [7168,8192] on zeros:
-// 1.97 PFLOP/s with the loads taken out, 1.79 with every second one, 1.42 with all of them (the eight-wave
-// 256 x 256 tile: 1.53; the vendor library: 2.25); on N(0, 0.02) data 1.29 against 1.36 and 1.63.  The
-// accumulators are pinned to the accumulation registers (Mfma::run_acc): left to the compiler, fragments of
-// the K loop are spilled around them and every reload waits for all loads in flight.
-template <class Cfg, int OP, int ODT>
-__device__ __attribute__((always_inline)) inline void big_tile_main(const GemmKArgs& p, IRIS_LDS char* lds) {
-  static_assert(Cfg::DMA && Cfg::LW == 0 && Cfg::KSUB == 1 && Cfg::S == 4 && Cfg::IM == Cfg::IN, "big-tile K loop");
-  constexpr int L = Cfg::L;
-  const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int lane = tid & 63;
-  int pid;
-  if (p.xcd_per > 0) {
-    const int x = blockIdx.x % p.num_xcds, j = blockIdx.x / p.num_xcds;
-    pid = j < p.xcd_per ? x * p.xcd_per + j : p.num_sms * 2;
-  } else {
-    pid = xcd_remap(blockIdx.x, p.num_sms, p.num_xcds);
-  }
-  const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
-  const int n_mine = pid < p.total_tiles ? (p.total_tiles - pid + p.num_sms - 1) / p.num_sms : 0;
-  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-  IRIS_LDS char* ws = lds + Cfg::S * Cfg::STAGE + wave * Cfg::WS_BYTES;
-  const int lrow = lane & 15, lq = lane >> 4;
-  const int xoff = (lq ^ ((lrow / Cfg::RP) % Cfg::CPR)) * 16;
-  const int a_off = (wm * Cfg::TM + lrow) * Cfg::BK * 2 + xoff;
-  const int b_off = Cfg::A_BYTES + (wn * Cfg::TN + lrow) * Cfg::BK * 2 + xoff;
-  const StreamRun sr{0, 0, 0};
-  Loader<Cfg> ld;
-  Frags<Cfg> fr;
-  f32x4 acc[Cfg::IM][Cfg::IN];
-
-  for (int t = 0; t < n_mine; ++t) {
-    const Item it = decode_item<Cfg, false>(p, sr, pid, t);
-    if (p.ts_begin && tid == 0)
-      __hip_atomic_fetch_min((IRIS_GLOBAL unsigned long long*)(p.ts_begin + it.tile_id),
-                             (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-    for (int i = 0; i < Cfg::IM; ++i)
-#pragma unroll
-      for (int j = 0; j < Cfg::IN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (nk > 0) {
-      // steps 0..3 into the four stages (steps past K fetch nothing)
-      ld.setup(p, it, wave, lane, 0);
-      ld.issue(p, lds, 0, wave);
-#pragma unroll
-      for (int s = 1; s < Cfg::S; ++s) {
-        ld.before_step(s, wave, lane);
-        ld.issue(p, lds + s * Cfg::STAGE, s, wave);
-      }
-      IRIS_WAIT_VMCNT(L * (Cfg::S - 1));
-      block_barrier_raw();
-      load_all<Cfg>(lds + a_off, lds + b_off, fr, 0);
-
-      auto step = [&](int g, auto par_tag) __attribute__((always_inline)) {
-        constexpr int cb = decltype(par_tag)::value;
-        mma_row<Cfg, false>(acc, fr, cb, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        // this wave's part of stage g+1 has landed (steps g+2 and g+3 may be in flight), and its reads of
-        // stage g, the fragments it is multiplying, have returned
-        IRIS_WAIT_VMCNT(L * (Cfg::S - 2));
-        IRIS_WAIT_LGKMCNT0();
-        block_barrier_raw();
-        const IRIS_LDS char* nst = lds + ((g + 1) & (Cfg::S - 1)) * Cfg::STAGE;
-        IRIS_LDS char* rst = lds + (g & (Cfg::S - 1)) * Cfg::STAGE;
-        ld.before_step(g + Cfg::S, wave, lane);
-        fr.a[0] = load_a<Cfg>(nst + a_off, 0);
-        fr.b[cb ^ 1][0] = load_b<Cfg>(nst + b_off, 0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 1; i < Cfg::IM; ++i) {
-          mma_row<Cfg, false>(acc, fr, cb, i);
-          fr.a[i] = load_a<Cfg>(nst + a_off, i);
-          fr.b[cb ^ 1][i] = load_b<Cfg>(nst + b_off, i);
-          // every wave is past its reads of stage g: refill it with step g+4, the loads shared out over the blocks
-#pragma unroll
-          for (int q = (i - 1) * L / (Cfg::IM - 1); q < i * L / (Cfg::IM - 1); ++q)
-            ld.issue_at(p, rst, g + Cfg::S, wave, q);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      };
-      int g = 0;
-      for (; g + 1 < nk; g += 2) {
-        step(g, std::integral_constant<int, 0>{});
-        step(g + 1, std::integral_constant<int, 1>{});
-      }
-      if (g < nk) step(g, std::integral_constant<int, 0>{});
-      // the last MFMAs' results must have left the matrix cores before they are read
-      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-    }
-    store_acc<Cfg, OP, ODT>(p, acc, ws, it.m0 + wm * Cfg::TM, it.n0 + wn * Cfg::TN, it.m_end, it.n_end, lane);
-    // this wave's stores have completed, none of its loads is still writing a stage, and it has read all it will
-    IRIS_WAIT_VMCNT(0);
-    IRIS_WAIT_LGKMCNT0();
-    __syncthreads();
-    if (p.flag_mode != 0 && wave == 0) publish_tile(p, it.tile_id, lane);
-    if (p.ts_end && tid == 0)
-      __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + it.tile_id),
-                             (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-}
-
-// The same tile with 64-deep stages and its prefetch staged in registers: whole 128-byte lines are fetched with
-// plain buffer loads into two sets of staging registers, a step and a half ahead and one load per block of
-// MFMAs over the whole step, and written into the LDS stage that the hand-over has just freed (two
-// ds_write_b128 per block of the step's second half).  The LDS layout is the DMA loader's, so the fragment
-// reads are the other tiles'.  The first two stages of a tile still come by LDS-DMA.
-template <class Cfg, int OP, int ODT>
-__device__ __attribute__((always_inline)) inline void big_tile_main_regs(const GemmKArgs& p, IRIS_LDS char* lds) {
-  static_assert(Cfg::DMA && Cfg::LW == 0 && Cfg::KSUB == 2 && Cfg::S == 2 && Cfg::IM == Cfg::IN && Cfg::IM == 8 &&
-                    Cfg::L == 16,
-                "register-staged K loop");
-  constexpr int L = Cfg::L;
-  const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int lane = tid & 63;
-  int pid;
-  if (p.xcd_per > 0) {
-    const int x = blockIdx.x % p.num_xcds, j = blockIdx.x / p.num_xcds;
-    pid = j < p.xcd_per ? x * p.xcd_per + j : p.num_sms * 2;
-  } else {
-    pid = xcd_remap(blockIdx.x, p.num_sms, p.num_xcds);
-  }
-  const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
-  const int n_mine = pid < p.total_tiles ? (p.total_tiles - pid + p.num_sms - 1) / p.num_sms : 0;
-  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-  IRIS_LDS char* ws = lds + Cfg::S * Cfg::STAGE + wave * Cfg::WS_BYTES;
-  const int lrow = lane & 15, lq = lane >> 4;
-  const int swz = (lrow / Cfg::RP) % Cfg::CPR;
-  const int x0 = (lq ^ swz) * 16, x1 = ((4 + lq) ^ swz) * 16;  // the lane's chunk of the two substeps
-  const int a_row = (wm * Cfg::TM + lrow) * Cfg::BK * 2;
-  const int b_row = Cfg::A_BYTES + (wn * Cfg::TN + lrow) * Cfg::BK * 2;
-  const int wdst = wave * 1024 + lane * 16;  // where this lane's 16 bytes of load 0 land in a stage
-  const StreamRun sr{0, 0, 0};
-  Loader<Cfg> ld;
-  Frags<Cfg> fr;
-  f32x4 acc[Cfg::IM][Cfg::IN];
-  u32x4 stg[2][L];
-
-  // Load i of K-step k into registers (the DMA loader's addresses).  Written as an instruction of its own:
-  // the compiler, tracking a builtin's result across the loop's back edge, waits for every load in flight at
-  // the top of each iteration, which takes the prefetch away; the waits before the registers are used are
-  // counted by hand below instead (the loads complete in the order they were issued).
-  typedef int i32x4 __attribute__((ext_vector_type(4)));
-  i32x4 da = {0, 0, 0, 0}, db = {0, 0, 0, 0};  // buffer descriptors of the tile's A and B panels
-  auto fetch = [&](int k, int i) __attribute__((always_inline)) -> u32x4 {
-    const bool isA = i < Cfg::A_LOADS;
-    const int j = isA ? i : i - Cfg::A_LOADS;
-    const uint32_t off = isA ? ld.va + (uint32_t)(j * ld.step_a) : ld.vb + (uint32_t)(j * ld.step_b);
-    const int soff = k * Cfg::BK * 2;
-    u32x4 v;
-    if (isA)
-      asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(v) : "v"(off), "s"(da), "s"(soff) : "memory");
-    else
-      asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(v) : "v"(off), "s"(db), "s"(soff) : "memory");
-    return v;
-  };
-  auto descriptor = [&](const char* base, uint32_t bytes) __attribute__((always_inline)) -> i32x4 {
-    const uint64_t b = (uint64_t)base;
-    return i32x4{(int)(uint32_t)b, (int)(uint32_t)((b >> 32) & 0xFFFF), (int)bytes, 0x00020000};
-  };
-  // ... and from registers into its place in `stage`
-  auto put = [&](IRIS_LDS char* stage, int i, const u32x4& v) __attribute__((always_inline)) {
-    const bool isA = i < Cfg::A_LOADS;
-    const int j = isA ? i : i - Cfg::A_LOADS;
-    *reinterpret_cast<IRIS_LDS u32x4*>(stage + (isA ? 0 : Cfg::A_BYTES) + j * Cfg::NL * 1024 + wdst) = v;
-  };
-
-  // The first two steps of a tile on their way, by LDS-DMA into the two stages: issued before the previous
-  // tile's epilogue, so that they land under it.  (Step 2 goes into the first set of staging registers when the
-  // tile starts: registers that the compiler may spill around the epilogue must not have loads in flight,
-  // which it does not know of.)
-  auto start_tile = [&](const Item& nx) __attribute__((always_inline)) {
-    ld.setup(p, nx, wave, lane, 0);
-    {
-      // (the same panels and bounds as the loader's descriptors)
-      const int m0c = min(nx.m0, p.M - 1), n0c = min(nx.n0, p.N - 1);
-      const int rows_a = nx.m0 < p.M ? min(Cfg::CM, p.M - nx.m0) : 0, rows_b = nx.n0 < p.N ? min(Cfg::CN, p.N - nx.n0) : 0;
-      da = descriptor(p.a + (int64_t)m0c * p.sam * 2,
-                      rows_a > 0 ? (uint32_t)(((int64_t)(rows_a - 1) * p.sam + p.K) * 2) : 0);
-      db = descriptor(p.b + (int64_t)n0c * p.sbn * 2,
-                      rows_b > 0 ? (uint32_t)(((int64_t)(rows_b - 1) * p.sbn + p.K) * 2) : 0);
-    }
-    ld.issue(p, lds, 0, wave);
-    ld.before_step(1, wave, lane);
-    ld.issue(p, lds + Cfg::STAGE, 1, wave);
-    ld.before_step(2, wave, lane);
-  };
-  Item it;
-  if (n_mine > 0) {
-    it = decode_item<Cfg, false>(p, sr, pid, 0);
-    if (nk > 0) start_tile(it);
-  }
-  for (int t = 0; t < n_mine; ++t) {
-#pragma unroll
-    for (int i = 0; i < Cfg::IM; ++i)
-#pragma unroll
-      for (int j = 0; j < Cfg::IN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    Item nx = it;
-    if (nk > 0) {
-      if constexpr (!Cfg::BIG_DMA) {
-#pragma unroll
-        for (int i = 0; i < L; ++i) stg[0][i] = fetch(2, i);
-      }
-      // (a later tile's first two steps were waited for with the previous tile's stores)
-      if (t == 0) IRIS_WAIT_VMCNT(Cfg::BIG_DMA ? 0 : L);  // the DMA loads are older than the register loads
-      block_barrier_raw();
-      load_all<Cfg>(lds + a_row + x0, lds + b_row + x0, fr, 0);
-
-      // step g; W: the staging set that holds step g+2 (the other one takes step g+3)
-      auto step = [&](int g, auto w_tag) __attribute__((always_inline)) {
-        constexpr int W = decltype(w_tag)::value;
-        IRIS_LDS char* stage = lds + (g & 1) * Cfg::STAGE;
-        const IRIS_LDS char* nst = lds + ((g + 1) & 1) * Cfg::STAGE;
-        ld.before_step(Cfg::BIG_DMA ? g + 2 : g + 3, wave, lane);
-        // first half: multiply the first 32 of K, fetch the fragments of the second 32
-        // (memory instructions between the MFMAs of a block, not behind them: a wave that issues several
-        // in a row lets its matrix core run dry meanwhile)
-#pragma unroll
-        for (int i = 0; i < Cfg::IM; ++i) {
-#pragma unroll
-          for (int j = 0; j < Cfg::IN; ++j) {
-            Mfma<Cfg::DT>::run_acc(fr.b[0][j], fr.a[i], acc[i][j]);
-            if (j == 1) {
-              fr.b[1][i] = load_b<Cfg>(stage + b_row + x1, i);
-              __builtin_amdgcn_sched_barrier(0);
-            }
-            if (j == 4 && !Cfg::BIG_DMA) {
-              stg[W ^ 1][i] = fetch(g + 3, i);
-              __builtin_amdgcn_sched_barrier(0);
-            }
-          }
-          fr.a[i] = load_a<Cfg>(stage + a_row + x1, i);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        // second half: hand-over, then the next stage's first fragments, and stage g refilled from registers
-        // (half of the first block's MFMAs cover the wait and the barrier, the other half the memory
-        // instructions right behind it)
-#pragma unroll
-        for (int j = 0; j < Cfg::IN / 2; ++j) Mfma<Cfg::DT>::run_acc(fr.b[1][j], fr.a[0], acc[0][j]);
-        __builtin_amdgcn_sched_barrier(0);
-        IRIS_WAIT_LGKMCNT0();  // this wave's reads of stage g and its writes of stage g+1 are done
-        if constexpr (Cfg::BIG_DMA) IRIS_WAIT_VMCNT(0);  // its part of stage g+1 has landed
-        block_barrier_raw();
-        // Block i puts loads 2i and 2i+1 of step g+2, issued a step ago.  Younger than load 2i+1 are the
-        // 14 - 2i that followed it then, this step's first eight and the i of its second half so far.
-        auto second_half = [&](auto ic) __attribute__((always_inline)) {
-          constexpr int i = decltype(ic)::value;
-          if constexpr (i == 0) {
-            fr.b[0][i] = load_b<Cfg>(nst + b_row + x0, i);
-            __builtin_amdgcn_sched_barrier(0);
-            Mfma<Cfg::DT>::run_acc(fr.b[1][4], fr.a[0], acc[0][4]);
-            if constexpr (Cfg::BIG_DMA) {
-              ld.issue_at(p, stage, g + 2, wave, 2 * i);
-            } else {
-              IRIS_WAIT_VMCNT(22 - i);
-              put(stage, 2 * i, stg[W][2 * i]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            Mfma<Cfg::DT>::run_acc(fr.b[1][5], fr.a[0], acc[0][5]);
-            if constexpr (Cfg::BIG_DMA)
-              ld.issue_at(p, stage, g + 2, wave, 2 * i + 1);
-            else
-              put(stage, 2 * i + 1, stg[W][2 * i + 1]);
-            __builtin_amdgcn_sched_barrier(0);
-            Mfma<Cfg::DT>::run_acc(fr.b[1][6], fr.a[0], acc[0][6]);
-            if constexpr (!Cfg::BIG_DMA) stg[W ^ 1][Cfg::IM + i] = fetch(g + 3, Cfg::IM + i);
-            __builtin_amdgcn_sched_barrier(0);
-            Mfma<Cfg::DT>::run_acc(fr.b[1][7], fr.a[0], acc[0][7]);
-            fr.a[i] = load_a<Cfg>(nst + a_row + x0, i);
-            __builtin_amdgcn_sched_barrier(0);
-          } else {
-#pragma unroll
-            for (int j = 0; j < Cfg::IN; ++j) {
-              Mfma<Cfg::DT>::run_acc(fr.b[1][j], fr.a[i], acc[i][j]);
-              if (j == 1) {
-                fr.b[0][i] = load_b<Cfg>(nst + b_row + x0, i);
-                __builtin_amdgcn_sched_barrier(0);
-              }
-              if (j == 3) {
-                if constexpr (Cfg::BIG_DMA) {
-                  ld.issue_at(p, stage, g + 2, wave, 2 * i);
-                } else {
-                  IRIS_WAIT_VMCNT(22 - i);
-                  put(stage, 2 * i, stg[W][2 * i]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-              }
-              if (j == 5) {
-                if constexpr (Cfg::BIG_DMA)
-                  ld.issue_at(p, stage, g + 2, wave, 2 * i + 1);
-                else
-                  put(stage, 2 * i + 1, stg[W][2 * i + 1]);
-                __builtin_amdgcn_sched_barrier(0);
-              }
-              if (j == 6 && !Cfg::BIG_DMA) {
-                stg[W ^ 1][Cfg::IM + i] = fetch(g + 3, Cfg::IM + i);
-                __builtin_amdgcn_sched_barrier(0);
-              }
-            }
-            fr.a[i] = load_a<Cfg>(nst + a_row + x0, i);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        };
-        second_half(std::integral_constant<int, 0>{});
-        second_half(std::integral_constant<int, 1>{});
-        second_half(std::integral_constant<int, 2>{});
-        second_half(std::integral_constant<int, 3>{});
-        second_half(std::integral_constant<int, 4>{});
-        second_half(std::integral_constant<int, 5>{});
-        second_half(std::integral_constant<int, 6>{});
-        second_half(std::integral_constant<int, 7>{});
-      };
-      int g = 0;
-      for (; g + 1 < nk; g += 2) {
-        step(g, std::integral_constant<int, 0>{});
-        step(g + 1, std::integral_constant<int, 1>{});
-      }
-      if (g < nk) step(g, std::integral_constant<int, 0>{});
-      // every wave is done with the stages (its reads, and its writes of the steps past the last, which are
-      // zeros): the next tile's first loads may go
-      IRIS_WAIT_LGKMCNT0();
-      block_barrier_raw();
-      if (t + 1 < n_mine) {
-        nx = decode_item<Cfg, false>(p, sr, pid, t + 1);
-        start_tile(nx);
-      }
-      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-    } else if (t + 1 < n_mine) {
-      nx = decode_item<Cfg, false>(p, sr, pid, t + 1);
-    }
-    store_acc<Cfg, OP, ODT>(p, acc, ws, it.m0 + wm * Cfg::TM, it.n0 + wn * Cfg::TN, it.m_end, it.n_end, lane);
-    IRIS_WAIT_VMCNT(0);
-    IRIS_WAIT_LGKMCNT0();
-    __syncthreads();
-    if (p.flag_mode != 0 && wave == 0) publish_tile(p, it.tile_id, lane);
-    it = nx;
-  }
-}
-
 // SPLIT: the split-K build of the kernel (only launched with p.split_k > 1);
 // the plain build carries none of its code or state.
 // FUSED: the one-shot epilogue as the reference program runs it
@@ -1417,17 +1046,6 @@ gemm_persistent_kernel(const GemmKArgs p) {
   static_assert(!MERGED || (!SPLIT && !FUSED), "blocks of the caller's tiles: the plain build only");
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   IRIS_LDS char* lds = (IRIS_LDS char*)lds_raw;
-  if constexpr (Cfg::IM * Cfg::IN * 4 > 128) {
-    static_assert(!SPLIT, "the 256-accumulator tiles have no split-K build");
-    if constexpr (!FUSED) {  // (no build with the reduce inside either)
-      if constexpr (Cfg::KSUB == 2)
-        big_tile_main_regs<Cfg, OP, ODT>(p, lds);
-      else
-        big_tile_main<Cfg, OP, ODT>(p, lds);
-    }
-    return;
-  }
-
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
@@ -1454,14 +1072,24 @@ gemm_persistent_kernel(const GemmKArgs p) {
   }
 
   constexpr bool split = SPLIT;
+  // The split build of a tile without the owner's hand-over only ever runs split-K proper (stream-K runs need
+  // the owner's way): one (tile, part) item per program.  Saying so at compile time takes the item loop, the
+  // load cursor's step into a next item and everything that would stay live across an epilogue for it
+  // (the next item's first fragments, the loader's state) out of these builds, whose registers are full.
+  constexpr bool ONE_ITEM = SPLIT && !Cfg::SPLIT_OWNER;
   const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
   const int work = split ? p.total_tiles * p.split_k : p.total_tiles;  // tiles, or (tile, part) pairs
   const int n_mine = pid < work ? (work - pid + p.num_sms - 1) / p.num_sms : 0;
   int n_items = split ? n_mine : n_mine * p.sub_m * p.sub_n;
   StreamRun sr{0, 0, 0};
   if constexpr (SPLIT) {
-    sr = p.stream_k ? stream_run(p, pid, nk) : split_run(p, pid, nk);
-    n_items = stream_items(sr, nk);
+    if constexpr (ONE_ITEM) {
+      sr = split_run(p, pid, nk);
+      n_items = stream_items(sr, nk) > 0 ? 1 : 0;
+    } else {
+      sr = p.stream_k ? stream_run(p, pid, nk) : split_run(p, pid, nk);
+      n_items = stream_items(sr, nk);
+    }
   }
   const int total_steps = n_items * nk;  // > 0 iff there is anything to load
 
@@ -1518,7 +1146,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
       pending_tile = -1;
     }
     if constexpr (SPLIT) {
-      if (p.sliced) {
+      if (ONE_ITEM || p.sliced) {
         // split-K proper: program pid is part pid % split_k of tile pid / split_k
         const int parts = p.split_k;
         const int slot0 = __builtin_amdgcn_readfirstlane((int)fast_div((uint32_t)pid, p.div_split) * parts);
@@ -1568,7 +1196,9 @@ gemm_persistent_kernel(const GemmKArgs p) {
         if (p.ts_end && tid == 0)
           __hip_atomic_fetch_max((IRIS_GLOBAL unsigned long long*)(p.ts_end + c_it.tile_id),
                                  (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, sr, pid, c_item);
+        if constexpr (!ONE_ITEM) {
+          if (++c_item < n_items) c_it = decode_item<Cfg, SPLIT>(p, sr, pid, c_item);
+        }
         return;
       }
       // (the tiles without the owner's way are only launched with the sliced one)
@@ -1674,7 +1304,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
     Item l_it;
     auto advance_load_cursor = [&]() __attribute__((always_inline)) {
       if (++l_k == l_kend) {
-        if (++l_item < n_items) {
+        if (!ONE_ITEM && ++l_item < n_items) {
           l_it = decode_item<Cfg, SPLIT>(p, sr, pid, l_item);
           const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, l_item, nk);
           l_k = kr.k_begin;
@@ -1841,14 +1471,20 @@ gemm_persistent_kernel(const GemmKArgs p) {
       }
     };
     int g = 0;
-    for (int it = 0; it < n_items; ++it) {
+    auto run_item = [&](int it) __attribute__((always_inline)) {
       stamp_begin();
       run_step(g, std::true_type{});
       ++g;
       const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, it, nk);
       const int steps = kr.k_end - kr.k_begin;
       for (int k = 1; k < steps; ++k, ++g) run_step(g, std::false_type{});
+      if constexpr (ONE_ITEM) IRIS_WAIT_VMCNT(0);  // (the loads past the last step fetch nothing, and nothing follows)
       epilogue();
+    };
+    if constexpr (ONE_ITEM) {
+      if (n_items > 0) run_item(0);
+    } else {
+      for (int it = 0; it < n_items; ++it) run_item(it);
     }
     IRIS_WAIT_VMCNT(0);  // no load may still be writing this group's LDS when it exits
   } else {

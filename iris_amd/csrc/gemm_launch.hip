@@ -524,14 +524,10 @@ hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan) {
     k.num_sms = 2 * a.num_sms;
     if (twin) plan->entry = twin;
   }
-  // A split launch of a 128-accumulator tile: the fetch state of the `_f4` build spills next
-  // to the hand-over's registers ([128,4096] x [4096,1376] as one 256 x 128 tile row in 16
-  // parts: 24.0 us against the plain tile's 21.2).
-  // Where the compiler puts those spills changes with unrelated edits: [8192,12288] x [12288,512] as 128
-  // tiles of 256 x 128 in two parts has run in 131 us (none inside the K loop) and in 181 (one fragment
-  // spilled and reloaded every K-step) with the `_f4` build, 158 with the plain one, which is what every
-  // such launch takes.  (The second launch of a split last round runs the `_f4` build: HBM bounds it.)
-  if (k.split_k != 1 && twin && !pick->split_owner && twin->bk == pick->bk) plan->entry = twin;
+  // (A split launch of a 128-accumulator tile runs the `_f4` build too: its split build handles one (tile, part)
+  // item per program and keeps nothing live across the epilogue, which leaves it 40 registers to spare.  Before
+  // that it spilled around the hand-over, now and then inside the K loop, and such launches took the plain tile:
+  // [8192,12288] x [12288,512] as 128 tiles of 256 x 128 in two parts 145 us, against 131 or 181 as the spills fell.)
   return hipSuccess;
 }
 

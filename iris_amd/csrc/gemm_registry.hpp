@@ -39,7 +39,7 @@ template <class Cfg, int OP, int ODT>
 constexpr GemmKernelFn fused_fn() {
   // (the tiles with fetching waves have no such build: the reduce wants the registers their
   // fetch state takes, and the launcher takes the plain tile of the same shape instead)
-  if constexpr ((OP == OP_STORE16 || OP == OP_STORE32) && Cfg::LW == 0 && Cfg::IM * Cfg::IN * 4 <= 128)
+  if constexpr ((OP == OP_STORE16 || OP == OP_STORE32) && Cfg::LW == 0)
     return &gemm_persistent_kernel<Cfg, OP, ODT, false, true>;
   else
     return nullptr;
@@ -80,8 +80,7 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 // and as deep a ring as LDS holds, since a fetching wave cannot refill the
 // stage that is being multiplied (256 x 64 tiles in three stages instead of
 // two: 57 -> 42 us on the same shape); and plain, which the launcher takes
-// where the first loses: with the reduce inside the program (no such build),
-// for a split launch of a 128-accumulator tile (its fetch state spills there),
+// where the first loses: with the reduce inside the program (no such build)
 // and for two programs per CU.
 #define IRIS_GEMM_VARIANTS(X, DT, OP)                                     \
   X(DT, OP, 256, 256, 64, 2, 4, 2, true, 0, 1, "256x256x64_w2x4_s2")         \
@@ -107,10 +106,7 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   X(DT, OP, 128, 256, 64, 2, 4, 2, true, 0, 1, "128x256x64_w2x4_s2")         \
   X(DT, OP, 128, 128, 32, 2, 2, 4, true, 0, 0, "128x128x32_w2x2_s4")         \
   X(DT, OP, 64, 64, 64, 2, 2, 4, true, 4, 1, "64x64x64_w2x2_s4_f4")          \
-  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")        \
-  X(DT, OP, 256, 256, 32, 2, 2, 4, true, 0, 0, "256x256x32_w2x2_s4")         \
-  X(DT, OP, 256, 256, 64, 2, 2, 2, true, 0, 0, "256x256x64_w2x2_s2_regs")    \
-  X(DT, OP, 256, 256, 64, 2, 2, 2, true, 1, 0, "256x256x64_w2x2_s2_dma")
+  X(DT, OP, 256, 64, 64, 4, 1, 2, true, 4, 1, "256x64x64_w4x1_s2_f4")
 
 #define IRIS_GEMM_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, SPLIT, NAME) \
   make_entry<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP>(NAME),
@@ -136,8 +132,6 @@ constexpr GemmKernelEntry make_entry(const char* name) {
 #define IRIS_GEMM_INSTANTIATE_FUSED_0(DT, OP, CM, CN, BK, WM, WN, S, DMA)                     \
   template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA>, OP, \
                                                   IRIS_GEMM_ODT(DT, OP), false, true>(const GemmKArgs);
-#define IRIS_GEMM_INSTANTIATE_FUSED_1(DT, OP, CM, CN, BK, WM, WN, S, DMA)
-#define IRIS_GEMM_INSTANTIATE_FUSED_2(DT, OP, CM, CN, BK, WM, WN, S, DMA)
 #define IRIS_GEMM_INSTANTIATE_FUSED_4(DT, OP, CM, CN, BK, WM, WN, S, DMA)
 
 // the store epilogues' builds whose tiles are blocks of the caller's

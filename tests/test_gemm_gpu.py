@@ -677,18 +677,21 @@ def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
         torch.cuda.synchronize()
         check_close(cg2, O.shard_gemm(A2, B2, dtype), f"256 x 256 tiles in {sk} parts")
         assert flags2.cpu().tolist()[:16] == [1] * 16 and int(locks.abs().max().item()) == 0
-    # a split 256 x 128 tile runs the plain build (the one with fetching waves spills around the hand-over)
-    for K3, name in ((8192, "256x128x64_w2x2_s2"), (4096, "256x128x64_w2x2_s2")):
+    # a split 256 x 128 tile runs the build with fetching waves, like an unsplit one; the plain build of the same
+    # tile (every wave fetches its share) has a split build too, reached by its variant number
+    plain = _variant_names().index("256x128x64_w2x2_s2") + 1
+    for K3, variant, name in ((8192, 0, "256x128x64_w2x2_s3_f4"), (4096, 0, "256x128x64_w2x2_s3_f4"),
+                              (4096, plain, "256x128x64_w2x2_s2")):
         A3, B3 = make_ab(512, 256, K3, dtype)
         a3, b3 = to_heap(shmem, A3), to_heap(shmem, B3)
         cg3 = shmem.zeros((512, 256), dtype=dtype)
         flags2.zero_()
         args3 = (a3, b3, None, cg3, flags2, None, 0, 1, 16, 256, 128, 64, 4, ops.EPI_ALL_SCATTER)
-        assert ops.gemm_split_k(*args3, partials=big, locks=locks) == 4
-        assert ops.gemm_plan_name(*args3, partials=big, locks=locks) == name
-        ops.gemm_launch(*args3, partials=big, locks=locks)
+        assert ops.gemm_split_k(*args3, partials=big, locks=locks, variant=variant) == 4
+        assert ops.gemm_plan_name(*args3, partials=big, locks=locks, variant=variant) == name
+        ops.gemm_launch(*args3, partials=big, locks=locks, variant=variant)
         torch.cuda.synchronize()
-        check_close(cg3, O.shard_gemm(A3, B3, dtype), f"256 x 128 tiles in 4 parts, K = {K3}")
+        check_close(cg3, O.shard_gemm(A3, B3, dtype), f"256 x 128 tiles in 4 parts, K = {K3}, {name}")
         assert flags2.cpu().tolist()[:4] == [1] * 4 and int(locks.abs().max().item()) == 0
 
 
