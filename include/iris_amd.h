@@ -137,6 +137,7 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 #define IRIS_GEMM_HANDOVER_AUTO 0
 #define IRIS_GEMM_HANDOVER_OWNER 1
 #define IRIS_GEMM_HANDOVER_SLICED 2
+#define IRIS_GEMM_HANDOVER_PAIR 3
 
 /*
  * Arguments of one persistent shard-GEMM launch.  It is the argument list of
@@ -187,8 +188,11 @@ typedef struct iris_gemm_args {
    * hand over to the tile's first part): IRIS_GEMM_HANDOVER_AUTO lets the
    * launcher decide, _OWNER: the first part adds the others' partials and runs
    * the epilogue, _SLICED: every part leaves its partial, then sums and stores
-   * its share of the tile's rows.  Both add the partials in part order: the
-   * results are bit-identical. */
+   * its share of the tile's rows, _PAIR (two parts of a 256 x 128, 128 x 256 or
+   * 256 x 256 compute tile only): each part keeps the accumulators of half the
+   * waves and leaves the other half's for the other part, so that slots of
+   * half a tile are enough.  All add the partials in part order: the results
+   * are bit-identical. */
   int32_t split_handover;
   int32_t flag_sem;     /* IRIS_FLAG_SEM_*: how a tile's flag orders its data                    */
 } iris_gemm_args;

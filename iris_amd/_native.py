@@ -28,7 +28,7 @@ SCOPE_AGENT, SCOPE_SYSTEM = 0, 1
 # special values of GemmArgs.variant (include/iris_amd.h)
 VARIANT_FEW_ROWS, VARIANT_PERSISTENT = 1000, 1001
 SPLIT_STREAM_K = -1  # GemmArgs.split_k: stream-K
-HANDOVER_AUTO, HANDOVER_OWNER, HANDOVER_SLICED = 0, 1, 2  # GemmArgs.split_handover
+HANDOVER_AUTO, HANDOVER_OWNER, HANDOVER_SLICED, HANDOVER_PAIR = 0, 1, 2, 3  # GemmArgs.split_handover
 # how a tile's flag orders its data (IRIS_FLAG_SEM_*)
 FLAG_SEM_WRITE_THROUGH, FLAG_SEM_RELEASE_ACQUIRE = 0, 1
 # status word (IRIS_STATUS_*)

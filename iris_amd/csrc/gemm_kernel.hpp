@@ -107,7 +107,7 @@ struct GemmKArgs {
   // runs the epilogue on them, so that no program does a whole tile's worth
   // of serial work; locks[first slot + 1] counts the parts that are done, and
   // the last one publishes the tile and re-arms both counters.
-  int sliced;
+  int sliced;  // 1: as above; 2 (two parts only): each part keeps the half of the waves it owns, see dump_half
   float* partials;
   int32_t* locks;
   int64_t partial_stride;
@@ -128,6 +128,17 @@ struct GemmKArgs {
   // merge_n of the caller's tiles; the flags stay the caller's, one per tile of BM / merge_m x BN / merge_n,
   // numbered over flag_num_pid_m x flag_num_pid_n tiles
   int merge_m, merge_n, flag_num_pid_m, flag_num_pid_n;
+
+  // L2 prefetch hints (tiles with fetching waves; 0: none).  The CUs of an XCD that work on one row of tiles
+  // share its A panel, those on one column of tiles its B panel, and a line that the first of them asks for comes
+  // from HBM while the others wait on the same miss.  With pf_dist > 0 a multiplying wave touches, every K-step,
+  // one dword of its share of the lines that step k + pf_dist will need (every pf_sa-th row of A, every pf_sb-th
+  // of B: the launch's tiles per XCD in either direction), so that the stage loads find them in L2.  Nothing
+  // depends on the loaded values.
+  int pf_dist, pf_sa, pf_sb;
+  // (MERGED builds) the launch covers the caller's columns of tiles from this one on: its flags sit that many
+  // columns to the right in the caller's grid of flag_num_pid_m x flag_num_pid_n tiles
+  int flag_pn_base;
 };
 
 template <int DT>
@@ -710,7 +721,7 @@ __device__ __attribute__((always_inline)) inline void publish_tile(const GemmKAr
   if constexpr (merged) {
     const TileCoord t = tile_map_fast(tile_id, p.num_pid_m, p.num_pid_n, p.G, p.tile_divs);
     pm0 = t.pid_m * p.merge_m;
-    pn0 = t.pid_n * p.merge_n;
+    pn0 = t.pid_n * p.merge_n + p.flag_pn_base;
     rows = min(p.merge_m, p.flag_num_pid_m - pm0);
     cols = min(p.merge_n, p.flag_num_pid_n - pn0);
   }
@@ -768,6 +779,41 @@ __device__ inline void add_partials(const GemmKArgs& p, f32x4 (&acc)[Cfg::IM][Cf
   for (int g = 0; g < GROUP; ++g)
 #pragma unroll
     for (int b = 0; b < NB; ++b) acc[b / Cfg::IN][b % Cfg::IN] += __builtin_bit_cast(f32x4, v[g][b]);
+}
+
+// Hand-over of a tile split in TWO parts: the first half of the multiplying waves belongs to part 0, the second
+// half to part 1.  A part leaves the accumulators of the waves that are NOT its own in its slot, in register
+// order (wave of the half, block, lane: 16 bytes a lane, 1 KiB a store), and each of its own waves adds what the
+// other part left for the same wave and runs the epilogue on its wave tile.  Half a partial tile crosses memory
+// per part, the other half never leaves its registers; p0 + p1 has the same bits whichever side adds.
+template <class Cfg>
+__device__ inline void dump_half(const GemmKArgs& p, const f32x4 (&acc)[Cfg::IM][Cfg::IN], int slot, int wv, int lane) {
+  constexpr int NB = Cfg::IM * Cfg::IN;
+  asm volatile("" : "+v"(lane));  // (offsets computed here, not kept in registers across the K loop)
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(p.partials + (int64_t)slot * p.partial_stride), 0, (Cfg::NW / 2) * NB * 1024, 0x00020000);
+#pragma unroll
+  for (int i = 0; i < Cfg::IM; ++i)
+#pragma unroll
+    for (int j = 0; j < Cfg::IN; ++j)
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rs,
+                                             ((wv * NB + i * Cfg::IN + j) * 64 + lane) * 16, 0, AUX_SC1);
+}
+template <class Cfg>
+__device__ inline void add_half(const GemmKArgs& p, f32x4 (&acc)[Cfg::IM][Cfg::IN], int slot, int wv, int lane) {
+  constexpr int NB = Cfg::IM * Cfg::IN, CH = NB < 8 ? NB : 8;  // blocks in flight
+  asm volatile("" : "+v"(lane));
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(p.partials + (int64_t)slot * p.partial_stride), 0, (Cfg::NW / 2) * NB * 1024, 0x00020000);
+#pragma unroll
+  for (int b0 = 0; b0 < NB; b0 += CH) {
+    u32x4 v[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c)  // sc1: coherent at agent scope without a fence
+      v[c] = __builtin_amdgcn_raw_buffer_load_b128(rs, ((wv * NB + b0 + c) * 64 + lane) * 16, 0, AUX_SC1);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) acc[(b0 + c) / Cfg::IN][(b0 + c) % Cfg::IN] += __builtin_bit_cast(f32x4, v[c]);
+  }
 }
 
 // Sliced hand-over, second half: rows [r0, r1) of the tile whose parts lie in
@@ -1043,7 +1089,7 @@ __device__ inline void fused_reduce_tile(const GemmKArgs& p, const Item& it, int
 template <class Cfg, int OP, int ODT, bool SPLIT = false, bool FUSED = false, bool MERGED = false>
 __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(Cfg::WPE, Cfg::WPE))) void
 gemm_persistent_kernel(const GemmKArgs p) {
-  static_assert(!MERGED || (!SPLIT && !FUSED), "blocks of the caller's tiles: the plain build only");
+  static_assert(!MERGED || !FUSED, "blocks of the caller's tiles: no build with the reduce inside");
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   IRIS_LDS char* lds = (IRIS_LDS char*)lds_raw;
   const int tid = threadIdx.x;
@@ -1132,11 +1178,46 @@ gemm_persistent_kernel(const GemmKArgs p) {
   Item c_it;
   if (n_items > 0) c_it = decode_item<Cfg, SPLIT>(p, sr, pid, 0);
 
+  // L2 prefetch hints (see GemmKArgs::pf_dist): the first two multiplying waves, one for A and one for B, hold a
+  // descriptor of the current tile's panel and each lane the offset of the row whose line it touches.
+  constexpr bool PF = Cfg::LW != 0 && Cfg::DMA && !FUSED;
+  __amdgpu_buffer_rsrc_t pf_rs = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, 0, 0x00020000);
+  uint32_t pf_off = 0x80000000u;
+  auto prefetch_setup = [&](const Item& it) __attribute__((always_inline)) {
+    if constexpr (PF) {
+      if (p.pf_dist > 0 && wave < 2) {
+        const bool isA = wave == 0;
+        const int origin = isA ? it.m0 : it.n0, extent = isA ? p.M : p.N, span = isA ? Cfg::CM : Cfg::CN;
+        const int64_t ld = isA ? p.sam : p.sbn;
+        const int rows = origin < extent ? min(span, extent - origin) : 0;
+        const char* base = (isA ? p.a : p.b) + (int64_t)min(origin, extent - 1) * ld * 2;
+        pf_rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, rows > 0 ? (int)(((int64_t)(rows - 1) * ld + p.K) * 2) : 0,
+                                                  0x00020000);
+        // this program's share: rows `first`, `first + share`, ... of the panel
+        const int share = isA ? p.pf_sa : p.pf_sb;
+        const int first = (isA ? it.ln0 / p.BN : it.lm0 / p.BM) % share;
+        const int row = first + share * lane;
+        pf_off = row < rows ? (uint32_t)((int64_t)row * ld * 2) : 0x80000000u;
+      }
+    }
+  };
+  // ... and touch the lines of K-step `k` (steps from `k_end` on are left alone).  The dword a lane fetches must
+  // land somewhere, and not in a register (the compiler would hand the register on before the load returns):
+  // it goes, by LDS-DMA, into the wave's own epilogue scratch, which nothing reads inside a K loop.  The last
+  // touch of a tile is issued pf_dist steps before its epilogue.
+  auto prefetch_step = [&](int k, int k_end) __attribute__((always_inline)) {
+    if constexpr (PF) {
+      if (p.pf_dist > 0 && wave < 2 && k < k_end)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(pf_rs, (IRIS_LDS void*)ws, 4, pf_off, k * Cfg::BK * 2, 0, 0);
+    }
+  };
+
   // end of a compute tile: store it, and publish the logical tile it completes
   // FUSED: a wait for a peer's tile has timed out.  The peer is not resident (or gone): the tiles that follow
   // are still stored and signalled, but not waited for, so that a launch without its peers costs one timeout
   // and not one per tile.
   int peers_gone = 0;
+  const GemmKArgs& p_outer = p;
   auto epilogue = [&]() __attribute__((always_inline)) {
     if (defer_publish && pending_tile >= 0) {
       // a one-step tile: the previous tile has not been published yet
@@ -1147,15 +1228,33 @@ gemm_persistent_kernel(const GemmKArgs p) {
     }
     if constexpr (SPLIT) {
       if (ONE_ITEM || p.sliced) {
+        // (One item per program: whatever this hand-over reads of the launch's arguments is read here, from the
+        // argument block, through a pointer the compiler cannot see through; held in scalar registers from the
+        // kernel's entry on, those arguments pushed fragments of the K loop out of the 128-accumulator tiles'
+        // registers: the split 256 x 256 tile stepped in 2.3 us instead of 1.5.)
+        typedef const __attribute__((address_space(4))) GemmKArgs* KernArgPtr;
+        KernArgPtr late_args = (KernArgPtr)__builtin_amdgcn_kernarg_segment_ptr();  // (the kernel's only parameter)
+        asm volatile("" : "+s"(late_args));
+        const GemmKArgs& p = ONE_ITEM ? *(const GemmKArgs*)late_args : p_outer;
         // split-K proper: program pid is part pid % split_k of tile pid / split_k
         const int parts = p.split_k;
         const int slot0 = __builtin_amdgcn_readfirstlane((int)fast_div((uint32_t)pid, p.div_split) * parts);
         const int part = pid - slot0;
         IRIS_LDS int* okslot = (IRIS_LDS int*)(lds + Cfg::S * Cfg::STAGE);  // wave 0's scratch, idle here
-        {
+        // two parts, each keeping the half of the waves it owns (see dump_half)
+        constexpr bool PAIR_BUILD = ONE_ITEM && Cfg::NW % 2 == 0;
+        const bool pair = PAIR_BUILD && p.sliced == 2;
+        const bool mine = (wave < Cfg::NW / 2) == (part == 0);
+        const int wv = wave < Cfg::NW / 2 ? wave : wave - Cfg::NW / 2;
+        if (pair) {
+          if constexpr (PAIR_BUILD) {
+            if (worker && !mine) dump_half<Cfg>(p, acc, pid, wv, lane);
+          }
+        } else {
           // the partial as a row-major [CM, CN] fp32 matrix in slot `pid`, through
           // the fp32 store epilogue (whole 128-byte lines, written through)
-          GemmKArgs q = p;
+          // (only what store_acc reads: a copy of all the arguments would be made in memory)
+          GemmKArgs q;
           q.out = (char*)(p.partials + (int64_t)pid * p.partial_stride);
           q.som = Cfg::CN;
           q.son = 1;
@@ -1163,6 +1262,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
           q.vec_out = 1;
           q.sys = 0;
           q.heap_bases = nullptr;
+          q.cur_rank = 0;
+          q.ws = 1;
           if (worker)
             store_acc<Cfg, OP_STORE32, IRIS_DTYPE_F32>(q, acc, ws, wm * Cfg::TM, wn * Cfg::TN, Cfg::CM, Cfg::CN, lane);
         }
@@ -1174,9 +1275,20 @@ gemm_persistent_kernel(const GemmKArgs p) {
         }
         __syncthreads();
         const int ok = *okslot;
-        if (ok && worker)
-          slice_epilogue<Cfg, OP, ODT>(p, c_it, slot0, parts, part * Cfg::CM / parts, (part + 1) * Cfg::CM / parts,
-                                       tid);
+        if (ok && worker) {
+          if (pair) {
+            if constexpr (PAIR_BUILD) {
+              if (mine) {
+                add_half<Cfg>(p, acc, slot0 + 1 - part, wv, lane);
+                store_acc<Cfg, OP, ODT>(p, acc, ws, c_it.m0 + wm * Cfg::TM, c_it.n0 + wn * Cfg::TN, c_it.m_end,
+                                        c_it.n_end, lane);
+              }
+            }
+          } else {
+            slice_epilogue<Cfg, OP, ODT>(p, c_it, slot0, parts, part * Cfg::CM / parts, (part + 1) * Cfg::CM / parts,
+                                         tid);
+          }
+        }
         IRIS_WAIT_VMCNT(0);  // this wave's stores of the slice have completed
         __syncthreads();     // (and okslot is scratch again)
         if (wave == 0 && ok) {
@@ -1236,6 +1348,12 @@ gemm_persistent_kernel(const GemmKArgs p) {
       static_assert(!SPLIT && (OP == OP_STORE16 || OP == OP_STORE32), "the in-program reduce follows a plain store");
       if (c_it.last_sub) {
         constexpr int IN_DT = OP == OP_STORE32 ? IRIS_DTYPE_F32 : ODT;
+        // (the arguments this part reads come from the argument block when it runs, not from registers held
+        // across the K loop: see the split hand-over above)
+        typedef const __attribute__((address_space(4))) GemmKArgs* KernArgPtr;
+        KernArgPtr late_args = (KernArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("" : "+s"(late_args));
+        const GemmKArgs& p = *(const GemmKArgs*)late_args;
         IRIS_LDS int* slot = (IRIS_LDS int*)(lds + Cfg::S * Cfg::STAGE);  // wave 0's scratch, idle by now
         IRIS_WAIT_VMCNT(0);  // this wave's stores of the partial tile have completed
         __syncthreads();
@@ -1473,11 +1591,16 @@ gemm_persistent_kernel(const GemmKArgs p) {
     int g = 0;
     auto run_item = [&](int it) __attribute__((always_inline)) {
       stamp_begin();
+      const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, it, nk);
+      prefetch_setup(c_it);
+      prefetch_step(kr.k_begin + p.pf_dist, kr.k_end);
       run_step(g, std::true_type{});
       ++g;
-      const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, it, nk);
       const int steps = kr.k_end - kr.k_begin;
-      for (int k = 1; k < steps; ++k, ++g) run_step(g, std::false_type{});
+      for (int k = 1; k < steps; ++k, ++g) {
+        prefetch_step(kr.k_begin + k + p.pf_dist, kr.k_end);
+        run_step(g, std::false_type{});
+      }
       if constexpr (ONE_ITEM) IRIS_WAIT_VMCNT(0);  // (the loads past the last step fetch nothing, and nothing follows)
       epilogue();
     };

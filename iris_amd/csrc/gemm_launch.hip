@@ -2,6 +2,7 @@
 #include <cstdio>
 #include <cstring>
 #include <cstdlib>
+#include <memory>
 #include <mutex>
 #include <utility>
 #include <vector>
@@ -63,6 +64,10 @@ struct Plan {
   // over the programs that round would leave idle
   int last_round = 0;
   GemmKArgs k_last{};
+  // the build that numbers its flags in a grid of its own (blocks of the caller's tiles, or a range of its columns)
+  int remap_flags = 0;
+  // a second plan behind this one: the columns of tiles this one leaves out
+  std::shared_ptr<Plan> rest;
 };
 
 int dbg() {
@@ -135,7 +140,7 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
   k.timeout = a.spin_timeout_ticks ? a.spin_timeout_ticks : 200000000ull;  // 2 s at 100 MHz
   k.stream_k = 0;
   if (a.split_k < 0 && a.split_k != IRIS_GEMM_SPLIT_STREAM_K) return hipErrorInvalidValue;
-  if (a.split_handover < IRIS_GEMM_HANDOVER_AUTO || a.split_handover > IRIS_GEMM_HANDOVER_SLICED)
+  if (a.split_handover < IRIS_GEMM_HANDOVER_AUTO || a.split_handover > IRIS_GEMM_HANDOVER_PAIR)
     return hipErrorInvalidValue;
   const int nk = (a.K + pick.bk - 1) / pick.bk;
   // the rules below were measured on K-steps of 64: `d` such steps to one of this tile
@@ -146,9 +151,14 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
   }
   if (a.split_k != 1 && a.partials && a.locks) {
     const bool resident = a.num_sms <= current_cu_count();
-    const bool possible = resident && pick.splitk && pick.fn_split && k.sub_m == 1 && k.sub_n == 1 &&
-                          a.partials_slot_elems >= (int64_t)pick.cm * pick.cn &&
-                          (reinterpret_cast<uintptr_t>(a.partials) & 15) == 0 && (a.partials_slot_elems % 4) == 0;
+    const bool any_way = resident && pick.splitk && pick.fn_split && k.sub_m == 1 && k.sub_n == 1 &&
+                         (reinterpret_cast<uintptr_t>(a.partials) & 15) == 0 && (a.partials_slot_elems % 4) == 0;
+    // Two parts of a 128-accumulator tile can meet with half a partial tile each (the pair hand-over: each part
+    // keeps the accumulators of the waves it owns), so a slot of half a tile is enough for them; that is what a
+    // caller who holds tiles half as wide has ([8192,14336] x [14336,448] in 256 x 64 tiles, run as 256 x 128).
+    const bool pair_ok = any_way && !pick.split_owner && (pick.wm * pick.wn) % 2 == 0 &&
+                         a.partials_slot_elems * 2 >= (int64_t)pick.cm * pick.cn;
+    const bool possible = any_way && a.partials_slot_elems >= (int64_t)pick.cm * pick.cn;
     // Stream-K: every program takes the same number of K-steps (within one).
     // A run of at least four steps keeps the parts of a tile few.
     const int64_t steps = (int64_t)k.total_tiles * nk;
@@ -159,10 +169,11 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
       if (!stream_ok) return hipErrorInvalidValue;
       k.stream_k = 1;
     } else if (a.split_k > 1) {
-      if (!possible || a.split_k > nk || a.split_k > 64 || (int64_t)k.total_tiles * a.split_k > a.num_sms)
+      if (!(possible || (pair_ok && a.split_k == 2)) || a.split_k > nk || a.split_k > 64 ||
+          (int64_t)k.total_tiles * a.split_k > a.num_sms)
         return hipErrorInvalidValue;
       k.split_k = a.split_k;
-    } else if (possible) {
+    } else if (possible || pair_ok) {
       if (k.total_tiles * 2 <= a.num_sms && nk * d >= 16) {
         // The hand-over of partials costs about as much as ten K-steps of a
         // small tile: as many parts as there are idle programs, at least four
@@ -173,6 +184,7 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
         int sk = a.num_sms / k.total_tiles;
         if (sk > nk * d / 4) sk = nk * d / 4;
         if (sk > 16) sk = 16;
+        if (!possible && sk > 2) sk = 2;  // (slots of half a tile: two parts)
         if (sk >= 4 || (sk > 1 && nk * d >= 32)) {
           k.split_k = sk;
         }
@@ -204,8 +216,16 @@ hipError_t plan_split(const iris_gemm_args& a, const GemmKernelEntry& pick, bool
     // (the 128-accumulator tiles only have the sliced one)
     if (a.split_handover == IRIS_GEMM_HANDOVER_SLICED && k.split_k > pick.cm) return hipErrorInvalidValue;
     if (a.split_handover == IRIS_GEMM_HANDOVER_OWNER && !pick.split_owner) return hipErrorInvalidValue;
+    const bool can_pair = k.split_k == 2 && !pick.split_owner && (pick.wm * pick.wn) % 2 == 0 &&
+                          a.partials_slot_elems * 2 >= (int64_t)pick.cm * pick.cn;
+    const bool can_slice = a.partials_slot_elems >= (int64_t)pick.cm * pick.cn;
+    if (a.split_handover == IRIS_GEMM_HANDOVER_PAIR && !can_pair) return hipErrorInvalidValue;
+    if (a.split_handover == IRIS_GEMM_HANDOVER_SLICED && !can_slice) return hipErrorInvalidValue;
+    // (two parts of a 128-accumulator tile: the pair hand-over moves half the bytes of the sliced one)
     k.sliced = a.split_handover == IRIS_GEMM_HANDOVER_SLICED  ? 1
                : a.split_handover == IRIS_GEMM_HANDOVER_OWNER ? 0
+               : a.split_handover == IRIS_GEMM_HANDOVER_PAIR  ? 2
+               : can_pair                                     ? 2
                                                               : (!pick.split_owner || k.split_k >= 8) ? 1 : 0;
   }
   if (k.stream_k) {
@@ -235,6 +255,32 @@ void launch_constants(const iris_gemm_args& a, const GemmKernelEntry& pick, Gemm
   k.part_major = (k.split_k > 1 && !k.stream_k && nk / k.split_k >= 32) ? k.total_tiles : 0;
   k.xcd_per = 0;
   if (!k.stream_k && a.num_xcds > 1 && work < a.num_sms) k.xcd_per = (int)((work + a.num_xcds - 1) / a.num_xcds);
+  // L2 prefetch hints for long walks over K (the tiles with fetching waves read them): an XCD's share of a round
+  // of tiles is a block of `rows` x `cols` neighbouring tiles, whose CUs share the A panels `cols` ways and the B
+  // panels `rows` ways.  They pay on the 64-column tiles, whose K-steps are short enough to be bound by how
+  // long a stage takes to arrive from HBM ([8192,14336] x [14336,448] in 256 x 64 tiles: 175 -> 161 us eight
+  // steps ahead, 155 sixteen ahead); the wider tiles' steps are bound by the matrix cores' power budget on real
+  // data and gain nothing (256 x 128: 427 -> 440 us on N(0, 0.02) data, 408 -> 380 us on zeros).
+  k.pf_dist = k.pf_sa = k.pf_sb = 0;
+  const int pf_dist = 8;
+  if (pick.fetch_waves > 0 && pick.cn <= 64 && !k.stream_k && k.sub_m == 1 && k.sub_n == 1 && nk >= 4 * pf_dist &&
+      a.num_xcds > 1) {
+    const int64_t per_xcd = k.xcd_per > 0 ? k.xcd_per : (k.num_sms / a.num_xcds);
+    int64_t tiles_per_xcd = k.split_k > 1 ? (per_xcd + k.split_k - 1) / k.split_k : per_xcd;
+    if (k.part_major > 0) tiles_per_xcd = per_xcd;  // (part by part: an XCD's programs are neighbouring tiles)
+    const int g_rows = k.G < k.num_pid_m ? k.G : k.num_pid_m;
+    int64_t cols = tiles_per_xcd / (g_rows > 0 ? g_rows : 1);
+    if (cols < 1) cols = 1;
+    if (cols > k.num_pid_n) cols = k.num_pid_n;
+    int64_t rows = tiles_per_xcd / cols;
+    if (rows < 1) rows = 1;
+    // one touch instruction per operand covers 64 rows of the share: the share must thin the panel out enough
+    if (cols * 64 >= pick.cm && rows * 64 >= pick.cn && cols * rows > 1) {
+      k.pf_dist = pf_dist;
+      k.pf_sa = (int)cols;
+      k.pf_sb = (int)rows;
+    }
+  }
 }
 
 // Validate `a` and build the launch plan.  Returns hipSuccess,
@@ -253,7 +299,7 @@ void split_last_round(const iris_gemm_args& a, Plan* plan) {
   const GemmKernelEntry* e = plan->entry;
   plan->last_round = 0;
   if (!e || plan->skinny || plan->in_program || k.split_k != 1 || k.stream_k || k.sub_m != 1 || k.sub_n != 1) return;
-  if (k.merge_m * k.merge_n > 1) return;  // (the split-K build raises one flag per tile of its own)
+  if (k.merge_m * k.merge_n > 1 || plan->remap_flags) return;  // (the second launch would raise flags of its own grid)
   if (a.split_k != 0 || a.variant != 0 || a.mm_begin_timestamp || a.mm_end_timestamp) return;
   if (!a.partials || !a.locks || !e->splitk || !e->fn_split || k.num_sms != a.num_sms) return;
   if (a.num_sms > current_cu_count() || a.partials_slot_elems < (int64_t)e->cm * e->cn) return;
@@ -279,6 +325,83 @@ void split_last_round(const iris_gemm_args& a, Plan* plan) {
   plan->last_round = 1;
 }
 
+// How a plain launch's tiles are blocked: merge_m x merge_n of the caller's tiles as one 256 x 256 or 256 x 128
+// tile, when the `tiles_n` columns of tiles suffice for it.  Returns false for "the caller's tiles as they are".
+bool choose_merge(const iris_gemm_args& a, int64_t tiles_n, int* merge_m, int* merge_n) {
+  *merge_m = *merge_n = 1;
+  const int64_t tiles_m = (a.M + a.block_m - 1) / a.block_m;
+  const int mm = 256 / a.block_m;  // 1 or 2
+  const int64_t rows = (tiles_m + mm - 1) / mm;
+  // 256 x 256 or 256 x 128, whichever finishes first among those that give (almost) every program a tile: rounds
+  // of tiles times the tile's time (a 256 x 256 tile does twice the work at 1.25 times the rate, as measured)
+  double best = 0;
+  for (int width = 256; width >= 128; width /= 2) {
+    const int mn = width / a.block_n;
+    const int64_t merged_tiles = rows * ((tiles_n + mn - 1) / mn);
+    // (seven programs in eight busy is enough: [8192,14336] x [14336,1792] as 224 tiles of 256 x 256 in one
+    // round against 448 of 256 x 128 in two)
+    if (mm * mn == 1 || merged_tiles * 8 < (int64_t)a.num_sms * 7) continue;
+    const double cost = (double)((merged_tiles + a.num_sms - 1) / a.num_sms) * (width == 256 ? 1.6 : 1.0);
+    if (best == 0 || cost < best) best = cost, *merge_m = mm, *merge_n = mn;
+  }
+  if (*merge_m * *merge_n > 1) return true;
+  if (!a.partials || !a.locks || a.K < 4096) return false;
+  // No block of the caller's tiles gives every program one.  Blocks that give every OTHER program one do, with
+  // each block's K range shared by two programs; their hand-over takes slots of half a (merged) tile, which is
+  // what the caller's workspace holds when the blocks are pairs of its tiles ([8192,14336] x [14336,448] in
+  // 256 x 64 tiles: 175 -> 114 us).
+  for (int width = 256; width >= 128; width /= 2) {
+    const int mn = width / a.block_n;
+    const int64_t merged_tiles = rows * ((tiles_n + mn - 1) / mn);
+    if (mm * mn == 1 || mn < 1) continue;
+    if (merged_tiles * 2 > a.num_sms || merged_tiles * 16 < (int64_t)a.num_sms * 7) continue;
+    if (a.partials_slot_elems * 2 < (int64_t)256 * width) continue;
+    *merge_m = mm, *merge_n = mn;
+    return true;
+  }
+  return false;
+}
+
+// The plan for the caller's tiles blocked merge_m x merge_n; false when the launcher has no kernel for it.
+bool plan_merged(const iris_gemm_args& a, int merge_m, int merge_n, Plan* plan) {
+  iris_gemm_args b = a;
+  b.block_m = a.block_m * merge_m;
+  b.block_n = a.block_n * merge_n;
+  Plan merged;
+  const hipError_t err = make_plan_body(b, &merged);
+  // (only the persistent kernels publish merged tiles: unsplit, or split in parts)
+  const bool unsplit = merged.k.split_k == 1 && merged.entry && merged.entry->fn_merged;
+  const bool parts = merged.k.split_k > 1 && merged.entry && merged.entry->fn_split_merged;
+  if (err != hipSuccess || !merged.entry || merged.skinny || !(unsplit || parts) || merged.k.stream_k || merged.in_program)
+    return false;
+  *plan = merged;
+  plan->remap_flags = 1;
+  plan->k.merge_m = merge_m;
+  plan->k.merge_n = merge_n;
+  plan->k.flag_num_pid_m = (a.M + a.block_m - 1) / a.block_m;
+  plan->k.flag_num_pid_n = (a.N + a.block_n - 1) / a.block_n;
+  plan->k.flag_pn_base = 0;
+  if (merge_m * merge_n > 1) split_last_round(b, plan);
+  return true;
+}
+
+// `a` restricted to columns [col0, col0 + cols) of B and of the output (whole tiles of the caller).
+iris_gemm_args column_range(const iris_gemm_args& a, int64_t col0, int64_t cols) {
+  iris_gemm_args b = a;
+  b.N = (int32_t)cols;
+  b.b = static_cast<const char*>(a.b) + col0 * a.stride_bn * 2;
+  if (a.epilogue == IRIS_EPI_ALL_SCATTER) {
+    // (the launcher adds cur_rank * N columns to c_global: of the range's N, so the difference goes in here;
+    // the pointer is only ever used with that offset added)
+    const int64_t shift = (int64_t)a.cur_rank * (a.N - cols) + col0;
+    b.c_global = static_cast<char*>(a.c_global) + shift * a.stride_cn_global * dtype_size(a.c_global_dtype);
+  } else {
+    b.c = static_cast<char*>(a.c) + col0 * a.stride_cn * dtype_size(a.c_dtype);
+    b.c_global = static_cast<char*>(a.c_global) + col0 * a.stride_cn_global * dtype_size(a.c_global_dtype);
+  }
+  return b;
+}
+
 // The plan of a launch.  A caller's tile that is narrow or short (the reference scripts' 256 x 64; 128 x 128)
 // makes a large GEMM wait for its operands: a 256 x 64 tile fetches 256 rows of A every K-step for 64 columns'
 // worth of work.  Where there are enough of them, the launch computes a block of the caller's tiles as one
@@ -286,48 +409,49 @@ void split_last_round(const iris_gemm_args& a, Plan* plan) {
 // computes a tile was never observable ([8192,8192] x [8192,1024] in 256 x 64 tiles: 739-762 -> 928 TFLOP/s
 // over the eight ranks of the reference's 07 benchmark).
 hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
-  int merge_m = 1, merge_n = 1;
   const bool plain = a.variant == 0 && a.split_k == 0 && !a.mm_begin_timestamp && !a.mm_end_timestamp &&
-                     !(a.epilogue == IRIS_EPI_ONE_SHOT && a.phase == IRIS_PHASE_FUSED) &&
+                     !(a.epilogue == IRIS_EPI_ONE_SHOT && a.phase != IRIS_PHASE_PRODUCE) &&
                      a.epilogue != IRIS_EPI_ATOMIC_ADD && a.num_sms > 0 && (a.block_m == 128 || a.block_m == 256) &&
                      (a.block_n == 64 || a.block_n == 128) && a.M >= 256;
-  if (plain) {
-    const int64_t tiles_m = (a.M + a.block_m - 1) / a.block_m, tiles_n = (a.N + a.block_n - 1) / a.block_n;
-    const int mm = 256 / a.block_m;  // 1 or 2
-    const int64_t rows = (tiles_m + mm - 1) / mm;
-    // 256 x 256 or 256 x 128, whichever finishes first among those that give every program a tile: rounds of
-    // tiles times the tile's time (a 256 x 256 tile does twice the work at 1.25 times the rate, as measured)
-    double best = 0;
-    for (int width = 256; width >= 128; width /= 2) {
-      const int mn = width / a.block_n;
-      const int64_t merged_tiles = rows * ((tiles_n + mn - 1) / mn);
-      if (mm * mn == 1 || merged_tiles < a.num_sms) continue;
-      const double cost = (double)((merged_tiles + a.num_sms - 1) / a.num_sms) * (width == 256 ? 1.6 : 1.0);
-      if (best == 0 || cost < best) best = cost, merge_m = mm, merge_n = mn;
-    }
-  }
-  if (merge_m * merge_n > 1) {
-    iris_gemm_args b = a;
-    b.block_m = a.block_m * merge_m;
-    b.block_n = a.block_n * merge_n;
-    Plan merged;
-    const hipError_t err = make_plan_body(b, &merged);
-    // (only the persistent kernels, unsplit, publish merged tiles)
-    if (err == hipSuccess && merged.entry && !merged.skinny && merged.k.split_k == 1 && !merged.k.stream_k &&
-        !merged.in_program && merged.entry->fn_merged) {
-      *plan = merged;
-      plan->k.merge_m = merge_m;
-      plan->k.merge_n = merge_n;
-      plan->k.flag_num_pid_m = (a.M + a.block_m - 1) / a.block_m;
-      plan->k.flag_num_pid_n = (a.N + a.block_n - 1) / a.block_n;
-      split_last_round(b, plan);
-      return hipSuccess;
+  const bool plain_two_kernels = a.variant == 0 && a.split_k == 0 && !a.mm_begin_timestamp && !a.mm_end_timestamp &&
+                                 a.epilogue == IRIS_EPI_ONE_SHOT && a.phase == IRIS_PHASE_TWO_KERNELS && a.num_sms > 0 &&
+                                 (a.block_m == 128 || a.block_m == 256) && (a.block_n == 64 || a.block_n == 128) &&
+                                 a.M >= 256;
+  if (plain || plain_two_kernels) {
+    const int64_t tiles_n = (a.N + a.block_n - 1) / a.block_n;
+    int merge_m = 1, merge_n = 1;
+    if (choose_merge(a, tiles_n, &merge_m, &merge_n)) {
+      if (plan_merged(a, merge_m, merge_n, plan)) return hipSuccess;
+    } else if (plain && a.N % a.block_n == 0) {
+      // The columns of tiles are one or a few too many for a blocking that pays: [8192,36864] x [36864,576] is nine
+      // columns of 256 x 64 tiles, eight of which block into 128 pairs with K in two parts.  The launch then
+      // takes the columns that block first and the remaining ones as a launch of their own behind it.
+      for (int width = 256; width >= 128; width /= 2) {
+        const int mn = width / a.block_n;
+        const int64_t main_n = tiles_n / mn * mn, rest_n = tiles_n - main_n;
+        if (mn < 2 || main_n == 0 || rest_n == 0 || rest_n * 4 > main_n) continue;
+        const iris_gemm_args am = column_range(a, 0, main_n * a.block_n);
+        if (!choose_merge(am, main_n, &merge_m, &merge_n)) continue;
+        Plan first;
+        if (!plan_merged(am, merge_m, merge_n, &first)) continue;
+        const iris_gemm_args ar = column_range(a, main_n * a.block_n, rest_n * a.block_n);
+        auto rest = std::make_shared<Plan>();
+        // (the remaining columns as the caller's tiles; their flags sit at their place in the caller's grid)
+        if (!plan_merged(ar, 1, 1, rest.get())) continue;
+        first.k.flag_num_pid_n = (int)tiles_n;
+        rest->k.flag_num_pid_n = (int)tiles_n;
+        rest->k.flag_pn_base = (int)main_n;
+        *plan = first;
+        plan->rest = rest;
+        return hipSuccess;
+      }
     }
   }
   const hipError_t err = make_plan_body(a, plan);
   plan->k.merge_m = plan->k.merge_n = 1;
   plan->k.flag_num_pid_m = plan->k.num_pid_m;
   plan->k.flag_num_pid_n = plan->k.num_pid_n;
+  plan->k.flag_pn_base = 0;
   if (err == hipSuccess) split_last_round(a, plan);
   return err;
 }
@@ -587,11 +711,13 @@ namespace {
 GemmKernelFn plan_fn(const Plan& plan) {
   const GemmKernelEntry* e = plan.entry;
   if (plan.in_program) return e->fn_fused;
-  if (plan.k.merge_m * plan.k.merge_n > 1) return e->fn_merged;
-  return (plan.k.split_k > 1 || plan.k.stream_k) ? e->fn_split : e->fn;
+  const bool split = plan.k.split_k > 1 || plan.k.stream_k;
+  if (plan.remap_flags) return split ? e->fn_split_merged : e->fn_merged;
+  return split ? e->fn_split : e->fn;
 }
 
-// Enqueue what `plan` describes on `stream`.
+// Enqueue what `plan` describes on `stream`.  (`args` is the caller's launch: only a reduce kernel behind the GEMM
+// reads it.)
 hipError_t run_plan(const Plan& plan, const iris_gemm_args& args, void* stream) {
   hipError_t err = hipSuccess;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -633,6 +759,10 @@ hipError_t run_plan(const Plan& plan, const iris_gemm_args& args, void* stream) 
       err = hipGetLastError();
       if (err != hipSuccess) return err;
     }
+  }
+  if (plan.rest) {
+    err = run_plan(*plan.rest, args, stream);
+    if (err != hipSuccess) return err;
   }
   if (plan.fused_reduce) {
     // The consumer half of the one-shot epilogue runs as a second kernel on
@@ -734,7 +864,10 @@ extern "C" int iris_gemm_launch_noalloc(const iris_gemm_args* args, void* stream
   // The array keeps what the last call left: the locks must start at zero (a
   // wait that timed out leaves one raised).  A fill kernel, not a memset, so
   // that the call can be recorded into a HIP graph.
-  const bool uses_locks = (plan.skinny && plan.k.flag_mode != 0) || (plan.entry && (plan.k.split_k > 1 || plan.k.stream_k || plan.last_round));
+  auto needs_locks = [](const Plan& q) {
+    return (q.skinny && q.k.flag_mode != 0) || (q.entry && (q.k.split_k > 1 || q.k.stream_k || q.last_round));
+  };
+  const bool uses_locks = needs_locks(plan) || (plan.rest && needs_locks(*plan.rest));
   if (uses_locks) {
     hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), a.locks, 0,
                        (int)(NOALLOC_LOCK_BYTES / sizeof(int32_t)));
@@ -797,6 +930,10 @@ extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t
   if (plan.last_round) {
     const size_t n = std::strlen(buf);
     std::snprintf(buf + n, len > n ? len - n : 0, "+last_round_in_%d_parts", plan.k_last.split_k);
+  }
+  if (plan.rest) {
+    const size_t n = std::strlen(buf);
+    std::snprintf(buf + n, len > n ? len - n : 0, "+last_%d_columns_apart", plan.rest->k.N);
   }
   return hipSuccess;
 }

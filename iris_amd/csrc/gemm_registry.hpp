@@ -24,6 +24,7 @@ struct GemmKernelEntry {
   GemmKernelFn fn_split;  // split-K build, or null
   GemmKernelFn fn_fused;  // build with the one-shot reduce inside the program (store epilogues), or null
   GemmKernelFn fn_merged;  // build whose tiles are blocks of the caller's (store epilogues, 256 x 128 and 256 x 256), or null
+  GemmKernelFn fn_split_merged;  // ... and its split-K build, or null
   const char* name;
 };
 
@@ -47,13 +48,23 @@ constexpr GemmKernelFn fused_fn() {
 
 // The launcher only merges the caller's tiles into 256 x 128 and 256 x 256 ones, for the store epilogues, and
 // runs them with the table's first tile of either shape.
+// (... and, for a range of the caller's columns launched on its own, with the 256 x 64 one as it is)
 template <class Cfg>
 constexpr bool merged_build = Cfg::CM == 256 && Cfg::DMA && Cfg::BK == 64 &&
-                              ((Cfg::CN == 256 && Cfg::LW == 0 && Cfg::NW == 8) || (Cfg::CN == 128 && Cfg::LW == 4));
+                              ((Cfg::CN == 256 && Cfg::LW == 0 && Cfg::NW == 8) || (Cfg::CN == 128 && Cfg::LW == 4) ||
+                               (Cfg::CN == 64 && Cfg::LW == 4 && Cfg::S == 3));
 template <class Cfg, int OP, int ODT>
 constexpr GemmKernelFn merged_fn() {
   if constexpr ((OP == OP_STORE16 || OP == OP_STORE32) && merged_build<Cfg>)
     return &gemm_persistent_kernel<Cfg, OP, ODT, false, false, true>;
+  else
+    return nullptr;
+}
+
+template <class Cfg, int OP, int ODT>
+constexpr GemmKernelFn split_merged_fn() {
+  if constexpr ((OP == OP_STORE16 || OP == OP_STORE32) && merged_build<Cfg> && Cfg::SPLITK)
+    return &gemm_persistent_kernel<Cfg, OP, ODT, true, false, true>;
   else
     return nullptr;
 }
@@ -64,7 +75,7 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   return GemmKernelEntry{Cfg::DT, OP,      Cfg::CM, Cfg::CN, Cfg::BK,        Cfg::WM,
                          Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::SPLIT_OWNER, Cfg::THREADS, Cfg::LW, Cfg::LDS_BYTES,
                          &gemm_persistent_kernel<Cfg, OP, ODT, false>, split_fn<Cfg, OP, ODT>(), fused_fn<Cfg, OP, ODT>(),
-                         merged_fn<Cfg, OP, ODT>(), name};
+                         merged_fn<Cfg, OP, ODT>(), split_merged_fn<Cfg, OP, ODT>(), name};
 }
 
 // The variants, in the launcher's order of preference: the first entry whose
@@ -139,7 +150,15 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 256, 64, 2, 4, 2, true, 0>, OP,                \
                                                   IRIS_GEMM_ODT(DT, OP), false, false, true>(const GemmKArgs); \
   template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 128, 64, 2, 2, 3, true, 4>, OP,                \
-                                                  IRIS_GEMM_ODT(DT, OP), false, false, true>(const GemmKArgs);
+                                                  IRIS_GEMM_ODT(DT, OP), false, false, true>(const GemmKArgs); \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 256, 64, 2, 4, 2, true, 0>, OP,                \
+                                                  IRIS_GEMM_ODT(DT, OP), true, false, true>(const GemmKArgs);  \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 128, 64, 2, 2, 3, true, 4>, OP,                \
+                                                  IRIS_GEMM_ODT(DT, OP), true, false, true>(const GemmKArgs);  \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 64, 64, 4, 1, 3, true, 4>, OP,                 \
+                                                  IRIS_GEMM_ODT(DT, OP), false, false, true>(const GemmKArgs); \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 64, 64, 4, 1, 3, true, 4>, OP,                 \
+                                                  IRIS_GEMM_ODT(DT, OP), true, false, true>(const GemmKArgs);
 
 #define IRIS_GEMM_DECLARE(TAG) const GemmKernelEntry* gemm_entries_##TAG(int* count);
 IRIS_GEMM_DECLARE(bf16_store16)

@@ -32,6 +32,7 @@ from ._native import (
     HANDOVER_AUTO,
     HANDOVER_OWNER,
     HANDOVER_SLICED,
+    HANDOVER_PAIR,
     FLAG_SEM_WRITE_THROUGH,
     FLAG_SEM_RELEASE_ACQUIRE,
 )

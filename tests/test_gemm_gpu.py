@@ -633,6 +633,102 @@ def test_split_k_all_scatter(shmem, M, N, K, BM, BN, split_k, dtype):
     assert torch.equal(got[ops.HANDOVER_AUTO].view(torch.int16), got[ops.HANDOVER_SLICED].view(torch.int16))
 
 
+@pytest.mark.parametrize("M,N,K,BM,BN,ws", [
+    (512, 256, 2048, 256, 128, 1),    # 256 x 128 with fetching waves: waves 0-1 are part 0's, 2-3 part 1's
+    (500, 300, 1032, 256, 256, 2),    # 256 x 256, eight waves, ragged edges and a ragged last K-step, two ranks
+    (256, 500, 640, 128, 256, 1),     # 128 x 256: the halves are column halves
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_split_k_in_two_parts_with_the_pair_hand_over(shmem, M, N, K, BM, BN, ws, dtype):
+    """Two parts of a 128-accumulator tile: each part keeps the accumulators of
+    the waves it owns and leaves the other half's in its slot, so slots of
+    HALF a tile are enough.  Bit-identical with the sliced hand-over (p0 + p1
+    either way); twice in a row: the locks are left re-armed."""
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((M, N * ws), dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total,), dtype=torch.int32)
+    grid = 16
+    full = shmem.zeros((grid, BM * BN), dtype=torch.float32)
+    half = shmem.zeros((grid, BM * BN // 2), dtype=torch.float32)  # what a caller with tiles half as wide holds
+    locks = shmem.zeros((grid,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+    for r in range(ws):
+        shmem.on_rank(cg, r).zero_()
+        shmem.on_rank(flags, r).zero_()
+    want = O.shard_gemm(A, B, dtype)
+    rank = ws - 1
+    args = (a, b, None, shmem.on_rank(cg, rank), shmem.on_rank(flags, rank), hb, rank, ws, grid, BM, BN, 64, 2,
+            ops.EPI_ALL_SCATTER)
+    got = {}
+    launch = 0
+    for name, P, handover in (("sliced", full, ops.HANDOVER_SLICED), ("pair", full, ops.HANDOVER_PAIR),
+                              ("pair, half slots", half, ops.HANDOVER_PAIR), ("auto, half slots", half, ops.HANDOVER_AUTO)):
+        for again in (1, 2):
+            launch += 1
+            for r in range(ws):
+                shmem.on_rank(cg, r).zero_()
+            ops.gemm_launch(*args, partials=P, locks=locks, split_k=2, split_handover=handover)
+            torch.cuda.synchronize()
+            for r in range(ws):
+                block = shmem.on_rank(cg, r)[:, rank * N:(rank + 1) * N]
+                check_close(block, want, f"{name}, launch {again}, rank {r}")
+                assert shmem.on_rank(flags, r).cpu().tolist() == [launch] * total
+            assert int(locks.abs().max().item()) == 0
+        got[name] = shmem.on_rank(cg, 0)[:, rank * N:(rank + 1) * N].cpu().clone()
+    for name in got:
+        assert torch.equal(got[name], got["sliced"]), name
+    # the sliced hand-over does not fit slots of half a tile, and a pair is two parts
+    with pytest.raises(ValueError):
+        ops.gemm_launch(*args, partials=half, locks=locks, split_k=2, split_handover=ops.HANDOVER_SLICED)
+    with pytest.raises(ValueError):
+        ops.gemm_launch(*args, partials=full, locks=locks, split_k=4, split_handover=ops.HANDOVER_PAIR)
+    assert ops.gemm_split_k(*args, partials=half, locks=locks, split_k=0) in (1, 2)  # never more with half slots
+
+
+@pytest.mark.parametrize("M,N,K,BM,BN,grid,kernel", [
+    # 2 x 7 tiles of 256 x 64 on 16 programs: 8 blocks of two tiles (the last one a single tile), K in two parts
+    (512, 448, 4096, 256, 64, 16, "256x128x64_w2x2_s3_f4+two_tiles_each"),
+    # 2 x 4 tiles of 256 x 128 on 8 programs: 4 blocks of two tiles as 256 x 256, K in two parts
+    (512, 512, 4096, 256, 128, 8, "256x256x64_w2x4_s2+two_tiles_each"),
+    # 2 x 3 tiles of 256 x 64, ragged in M and N, on 8 programs: 2 x 2 blocks, the last column a single narrow tile
+    (500, 180, 4096, 256, 64, 8, "256x128x64_w2x2_s3_f4+two_tiles_each"),
+    # 2 x 9 tiles of 256 x 64 on 16 programs: the first eight columns as 8 blocks with K in two parts, then the
+    # ninth as a launch of its own (2 tiles, K in eight parts), whose flags sit in the caller's ninth column
+    (512, 576, 4096, 256, 64, 16, "256x128x64_w2x2_s3_f4+two_tiles_each+last_64_columns_apart"),
+])
+def test_blocks_of_the_callers_tiles_with_k_in_two_parts(shmem, M, N, K, BM, BN, grid, kernel):
+    """Too few blocks of the caller's tiles for every program, but enough for
+    every other one: each block's K range is shared by two programs, whose
+    hand-over fits the caller's workspace (slots of one of ITS tiles).  Every
+    tile of the caller keeps its id and its flag."""
+    dtype, ws = torch.bfloat16, 2
+    A, B = make_ab(M, N, K, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.zeros((M, N * ws), dtype=dtype)
+    total = ops.cdiv(M, BM) * ops.cdiv(N, BN)
+    flags = shmem.zeros((total + 2,), dtype=torch.int32)
+    partials, locks = split_workspace(shmem, grid, BM, BN)
+    hb = shmem.get_heap_bases()
+    for r in range(ws):
+        shmem.on_rank(cg, r).zero_()
+        shmem.on_rank(flags, r).zero_()
+    args = (a, b, None, shmem.on_rank(cg, 1), shmem.on_rank(flags, 1), hb, 1, ws, grid, BM, BN, 64, 1, ops.EPI_ALL_SCATTER)
+    assert ops.gemm_plan_name(*args, partials=partials, locks=locks) == kernel
+    assert ops.gemm_split_k(*args, partials=partials, locks=locks) == 2
+    assert ops.gemm_split_k(*args) == 1  # no workspace: the caller's tiles, unsplit
+    want = O.shard_gemm(A, B, dtype)
+    for launch in (1, 2):
+        ops.gemm_launch(*args, partials=partials, locks=locks)
+        torch.cuda.synchronize()
+        for r in range(ws):
+            check_close(shmem.on_rank(cg, r)[:, N:], want, f"launch {launch}, rank {r}")
+            assert shmem.on_rank(flags, r).cpu().tolist() == [launch] * total + [0, 0]
+            assert float(shmem.on_rank(cg, r)[:, :N].float().abs().max()) == 0.0  # rank 0's columns untouched
+        assert int(locks.abs().max().item()) == 0
+
+
 def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
     dtype = torch.bfloat16
     A, B = make_ab(72, 1376, 4096, dtype)  # (up to 64 rows would go to the few-rows kernel)
@@ -697,9 +793,12 @@ def test_split_k_is_chosen_for_few_tiles_and_long_k_only(shmem):
 
 @pytest.mark.parametrize("M,N,BN,ws,suffix", [
     # 18 tiles on 16 programs: 16 whole, 2 in four parts (the owner's hand-over)
-    (512, 576, 64, 1, "256x64x64_w4x1_s3_f4+last_round_in_4_parts"),
+    (1536, 192, 64, 1, "256x64x64_w4x1_s3_f4+last_round_in_4_parts"),
     # 18 tiles: 16 whole, 2 in four parts (the sliced hand-over), on two ranks
-    (512, 1152, 128, 2, "256x128x64_w2x2_s3_f4+last_round_in_4_parts"),
+    (1536, 384, 128, 2, "256x128x64_w2x2_s3_f4+last_round_in_4_parts"),
+    # nine columns of tiles: eight of them in blocks of two tiles with K in two parts, the ninth as a launch of its own
+    (512, 576, 64, 1, "256x128x64_w2x2_s3_f4+two_tiles_each+last_64_columns_apart"),
+    (512, 1152, 128, 2, "256x256x64_w2x4_s2+two_tiles_each+last_128_columns_apart"),
 ])
 def test_a_short_last_round_of_long_tiles_is_split_over_the_idle_programs(shmem, M, N, BN, ws, suffix):
     """Tiles a few more than a multiple of the programs, K long: the full rounds
@@ -722,7 +821,7 @@ def test_a_short_last_round_of_long_tiles_is_split_over_the_idle_programs(shmem,
         args = (a, bs[r], None, shmem.on_rank(cg, r), shmem.on_rank(flags, r), hb, r, ws, grid, 256, BN, 64, 4,
                 ops.EPI_ALL_SCATTER)
         assert ops.gemm_plan_name(*args, partials=partials, locks=locks) == suffix
-        assert "last_round" not in ops.gemm_plan_name(*args)                    # no workspace: as before
+        assert "last_" not in ops.gemm_plan_name(*args)                         # no workspace: as before
         ops.gemm_launch(*args, partials=partials, locks=locks)
         torch.cuda.synchronize()
         assert int(locks.abs().max().item()) == 0
@@ -731,16 +830,21 @@ def test_a_short_last_round_of_long_tiles_is_split_over_the_idle_programs(shmem,
         check_close(shmem.on_rank(cg, r), want, f"rank {r}")
         assert shmem.on_rank(flags, r).cpu().tolist() == [ws] * total + [0] * 3
     # a shorter K keeps the one launch
-    assert "last_round" not in ops.gemm_plan_name(a[:, :2048], bs[0][:2048], None, cg, flags, hb, 0, ws, grid, 256, BN, 64,
+    assert "last_" not in ops.gemm_plan_name(a[:, :2048], bs[0][:2048], None, cg, flags, hb, 0, ws, grid, 256, BN, 64,
                                                   4, ops.EPI_ALL_SCATTER, partials=partials, locks=locks)
 
 
-def test_split_last_round_with_the_one_shot_producer_and_reduce(shmem):
+@pytest.mark.parametrize("M,N,plan", [
+    # 16 whole tiles, then the last two in four parts
+    (1536, 192, "256x64x64_w4x1_s3_f4+last_round_in_4_parts"),
+    # eight columns of tiles in blocks of two with K in two parts, then the ninth column
+    (512, 576, "256x128x64_w2x2_s3_f4+two_tiles_each+last_64_columns_apart"),
+])
+def test_split_last_round_with_the_one_shot_producer_and_reduce(shmem, M, N, plan):
     """K-shards on two ranks, 18 tiles of 256 x 64 on 16 programs, K = 8192 a rank:
-    each producer is two launches (16 whole tiles, then the last two in four
-    parts), the fp32 partials and the flags on the other rank are as from one
-    launch, and the reduce gives the oracle's sum."""
-    ws, M, N, dtype, grid = 2, 512, 576, torch.bfloat16, 16
+    each producer is two launches, the fp32 partials and the flags on the other
+    rank are as from one launch, and the reduce gives the oracle's sum."""
+    ws, dtype, grid = 2, torch.bfloat16, 16
     K = 8192 * ws
     A, B = make_ab(M, N, K, dtype)
     shards = O.k_shards(A, B, ws)
@@ -759,7 +863,7 @@ def test_split_last_round_with_the_one_shot_producer_and_reduce(shmem):
         args = (ah[:, r * kk:(r + 1) * kk], bh[r * kk:(r + 1) * kk, :], shmem.on_rank(part, r), shmem.on_rank(out, r),
                 shmem.on_rank(flags, r), hb, r, ws, grid, 256, 64, 64, 6, ops.EPI_ONE_SHOT)
         kw = dict(phase=ops.PHASE_PRODUCE, partials=partials, locks=locks)
-        assert ops.gemm_plan_name(*args, **kw) == "256x64x64_w4x1_s3_f4+last_round_in_4_parts"
+        assert ops.gemm_plan_name(*args, **kw) == plan
         ops.gemm_launch(*args, **kw)
         torch.cuda.synchronize()
         assert int(locks.abs().max().item()) == 0
