@@ -178,11 +178,12 @@ def steady_ms(fn, settle_s=0.2, n=200):
     return s.elapsed_time(e) / n
 
 
-def graph_ms(fn, per_graph=20, replays=20):
+def graph_ms(fn, per_graph=20, replays=20, settle_s=0.02, batches=3):
     """Mean device ms per call of `fn`, with `per_graph` calls captured in a HIP
     graph so that the host's launch cost (tens of microseconds per call through
     Python) does not bound what is measured.  The launchers only enqueue
-    kernels on the current stream, so they can be captured."""
+    kernels on the current stream, so they can be captured.  Median of
+    `batches` timed batches after a short settle phase."""
     import torch
 
     side = torch.cuda.Stream()
@@ -195,16 +196,23 @@ def graph_ms(fn, per_graph=20, replays=20):
     with torch.cuda.graph(graph):
         for _ in range(per_graph):
             fn()
-    for _ in range(3):
-        graph.replay()
-    torch.cuda.synchronize()
+    # Settle first: after an idle period the power management lets the first launches run fast and then clamps
+    # the clocks for a few milliseconds, which a measurement of a few hundred microseconds would catch at random.
+    t_end = time.perf_counter() + settle_s
+    while time.perf_counter() < t_end:
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
     s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    s.record()
-    for _ in range(replays):
-        graph.replay()
-    e.record()
-    torch.cuda.synchronize()
-    return s.elapsed_time(e) / (per_graph * replays)
+    times = []
+    for _ in range(batches):
+        s.record()
+        for _ in range(replays):
+            graph.replay()
+        e.record()
+        torch.cuda.synchronize()
+        times.append(s.elapsed_time(e) / (per_graph * replays))
+    return statistics.median(times)
 
 
 def context_figures(a, b, c_global, flops, gemm_on):

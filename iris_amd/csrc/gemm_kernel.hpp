@@ -129,7 +129,7 @@ struct GemmKArgs {
   // numbered over flag_num_pid_m x flag_num_pid_n tiles
   int merge_m, merge_n, flag_num_pid_m, flag_num_pid_n;
 
-  // L2 prefetch hints (tiles with fetching waves; 0: none).  The CUs of an XCD that work on one row of tiles
+  // L2 prefetch hints (the 256 x 64 tile with fetching waves; 0: none).  The CUs of an XCD that work on one row of tiles
   // share its A panel, those on one column of tiles its B panel, and a line that the first of them asks for comes
   // from HBM while the others wait on the same miss.  With pf_dist > 0 a multiplying wave touches, every K-step,
   // one dword of its share of the lines that step k + pf_dist will need (every pf_sa-th row of A, every pf_sb-th
@@ -1180,7 +1180,9 @@ gemm_persistent_kernel(const GemmKArgs p) {
 
   // L2 prefetch hints (see GemmKArgs::pf_dist): the first two multiplying waves, one for A and one for B, hold a
   // descriptor of the current tile's panel and each lane the offset of the row whose line it touches.
-  constexpr bool PF = Cfg::LW != 0 && Cfg::DMA && !FUSED;
+  // (compiled into the 256 x 64 tile only: a test and a branch per K-step are felt by the small tiles, whose
+  // steps take 0.2 us: [512,4096] x [4096,1376] in 64 x 64 x 128 tiles 19.9 -> 24.3 us)
+  constexpr bool PF = Cfg::LW != 0 && Cfg::DMA && !FUSED && Cfg::CM == 256 && Cfg::CN == 64;
   __amdgpu_buffer_rsrc_t pf_rs = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, 0, 0x00020000);
   uint32_t pf_off = 0x80000000u;
   auto prefetch_setup = [&](const Item& it) __attribute__((always_inline)) {

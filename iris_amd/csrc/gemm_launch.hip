@@ -263,7 +263,7 @@ void launch_constants(const iris_gemm_args& a, const GemmKernelEntry& pick, Gemm
   // data and gain nothing (256 x 128: 427 -> 440 us on N(0, 0.02) data, 408 -> 380 us on zeros).
   k.pf_dist = k.pf_sa = k.pf_sb = 0;
   const int pf_dist = 8;
-  if (pick.fetch_waves > 0 && pick.cn <= 64 && !k.stream_k && k.sub_m == 1 && k.sub_n == 1 && nk >= 4 * pf_dist &&
+  if (pick.fetch_waves > 0 && pick.cm == 256 && pick.cn == 64 && !k.stream_k && k.sub_m == 1 && k.sub_n == 1 && nk >= 16 * pf_dist &&
       a.num_xcds > 1) {
     const int64_t per_xcd = k.xcd_per > 0 ? k.xcd_per : (k.num_sms / a.num_xcds);
     int64_t tiles_per_xcd = k.split_k > 1 ? (per_xcd + k.split_k - 1) / k.split_k : per_xcd;
