@@ -117,8 +117,8 @@ def main(algorithm, argv=None):
             args["gemm_sms"] = fit
 
     datatype = DATATYPES[args["datatype"]]
-    if datatype not in (torch.float16, torch.bfloat16):
-        print(f"Datatype {args['datatype']} is not supported by the HIP kernels (fp16 and bf16 are).")
+    if datatype not in (torch.float16, torch.bfloat16, torch.float32):
+        print(f"Datatype {args['datatype']} is not supported by the HIP kernels (fp16, bf16 and fp32 are).")
         sys.exit(1)
 
     assert args["n"] % world_size == 0, f"N ({args['n']}) must be divisible by world size ({world_size})."

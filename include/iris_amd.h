@@ -164,7 +164,7 @@ typedef struct iris_gemm_args {
   int32_t num_sms;      /* NUM_SMS == grid size                         gemm_*:120 */
   int32_t num_xcds;     /* NUM_XCDS                                     gemm_*:122 */
   int32_t cur_rank, world_size; /*                                      gemm_*:126-127 */
-  int32_t ab_dtype;     /* IRIS_DTYPE_F16 | IRIS_DTYPE_BF16                       */
+  int32_t ab_dtype;     /* IRIS_DTYPE_F16 | IRIS_DTYPE_BF16; IRIS_DTYPE_F32 with fp32 outputs */
   int32_t c_dtype;      /* element type of c                                      */
   int32_t c_global_dtype; /* element type of c_global                             */
   int32_t epilogue;     /* IRIS_EPI_*                                             */

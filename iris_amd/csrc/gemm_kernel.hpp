@@ -158,6 +158,22 @@ struct Mfma<IRIS_DTYPE_F16> {
   }
 };
 
+// fp32 operands.  The launcher hands such a launch over with K and the operands' strides counted in 16-bit units
+// (two to an element), so that slabs, stages and loaders are the 16-bit kernels' byte for byte: a 16-byte chunk of a
+// slab row holds four elements where it held eight.  A lane's fragment of a 32-unit substep is then four
+// consecutive k of its row, and the substep's product is four v_mfma_f32_16x16x4_f32, the e-th over the lanes' e-th
+// elements: lane group g contributes k = 4 g + e, so the four cover the substep's sixteen k once each (operands A
+// and B pair up the same way, which is all a sum over k asks for).
+template <>
+struct Mfma<IRIS_DTYPE_F32> {
+  using vec8 = f32x4;
+  __device__ static inline f32x4 run(vec8 a, vec8 b, f32x4 c) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], c, 0, 0, 0);
+    return c;
+  }
+};
+
 // LW_: waves that only fetch.  With one wave per SIMD a wave that is held up
 // at the issue of a load (the memory pipeline takes a wave's loads at the
 // rate it delivers them) runs no MFMA meanwhile, and the K loop costs the sum
@@ -428,12 +444,14 @@ __device__ inline void load_slab_generic(const GemmKArgs& p, const Item& it, IRI
         const int kk = k0 + ch * 8 + e * 2 + h;
         unsigned short x = 0;
         if (kk < p.K) {
+          // (fp32 operands: 16-bit unit kk is half kk & 1 of element kk / 2, and the strides count units)
+          const int64_t ke = Cfg::DT == IRIS_DTYPE_F32 ? kk >> 1 : kk, half = Cfg::DT == IRIS_DTYPE_F32 ? kk & 1 : 0;
           if (isA) {
             const int r = min(it.m0 + row, p.M - 1);
-            x = A[(int64_t)r * p.sam + (int64_t)kk * p.sak];
+            x = A[(int64_t)r * p.sam + ke * p.sak + half];
           } else {
             const int r = min(it.n0 + row, p.N - 1);
-            x = B[(int64_t)r * p.sbn + (int64_t)kk * p.sbk];
+            x = B[(int64_t)r * p.sbn + ke * p.sbk + half];
           }
         }
         w |= ((unsigned int)x) << (16 * h);

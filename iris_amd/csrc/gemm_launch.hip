@@ -28,6 +28,11 @@ const GemmKernelEntry* entries_for(int dt, int op, int* count) {
       case OP_ATOMIC32: return gemm_entries_f16_atomic32(count);
       case OP_ATOMIC16: return gemm_entries_f16_atomic16(count);
     }
+  } else if (dt == IRIS_DTYPE_F32) {
+    switch (op) {
+      case OP_STORE32: return gemm_entries_f32_store32(count);
+      case OP_ATOMIC32: return gemm_entries_f32_atomic32(count);
+    }
   }
   *count = 0;
   return nullptr;
@@ -408,7 +413,25 @@ iris_gemm_args column_range(const iris_gemm_args& a, int64_t col0, int64_t cols)
 // 256 x 128 or 256 x 256 tile and raises each one's flag: tile ids and flags are the caller's, which program
 // computes a tile was never observable ([8192,8192] x [8192,1024] in 256 x 64 tiles: 739-762 -> 928 TFLOP/s
 // over the eight ranks of the reference's 07 benchmark).
+hipError_t make_plan_units(const iris_gemm_args& a, Plan* plan);
+
+// fp32 operands (the reference scripts' --datatype fp32; the output is fp32 too): the kernels count K and the
+// operands' strides in 16-bit units, two to an element, and everything between this function and the MFMAs
+// (loaders, slabs, stages, K tail, the 2 GiB windows of the buffer descriptors) is the 16-bit kernels' as it is.
 hipError_t make_plan(const iris_gemm_args& a, Plan* plan) {
+  if (a.ab_dtype != IRIS_DTYPE_F32) return make_plan_units(a, plan);
+  const int64_t lim = (int64_t)1 << 30;
+  if (a.K < 0 || a.K >= lim) return hipErrorInvalidValue;
+  iris_gemm_args b = a;
+  b.K = 2 * a.K;
+  b.stride_am = 2 * a.stride_am;
+  b.stride_ak = 2 * a.stride_ak;
+  b.stride_bk = 2 * a.stride_bk;
+  b.stride_bn = 2 * a.stride_bn;
+  return make_plan_units(b, plan);
+}
+
+hipError_t make_plan_units(const iris_gemm_args& a, Plan* plan) {
   const bool plain = a.variant == 0 && a.split_k == 0 && !a.mm_begin_timestamp && !a.mm_end_timestamp &&
                      !(a.epilogue == IRIS_EPI_ONE_SHOT && a.phase != IRIS_PHASE_PRODUCE) &&
                      a.epilogue != IRIS_EPI_ATOMIC_ADD && a.num_sms > 0 && (a.block_m == 128 || a.block_m == 256) &&
@@ -462,7 +485,8 @@ hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan) {
   if (a.num_sms <= 0 || a.num_xcds <= 0 || (a.num_sms % a.num_xcds) != 0) return hipErrorInvalidValue;
   if (a.world_size <= 0 || a.cur_rank < 0 || a.cur_rank >= a.world_size) return hipErrorInvalidValue;
   if (a.world_size > 1 && a.heap_bases == nullptr) return hipErrorInvalidValue;
-  if (a.ab_dtype != IRIS_DTYPE_BF16 && a.ab_dtype != IRIS_DTYPE_F16) return hipErrorInvalidValue;
+  if (a.ab_dtype != IRIS_DTYPE_BF16 && a.ab_dtype != IRIS_DTYPE_F16 && a.ab_dtype != IRIS_DTYPE_F32)
+    return hipErrorInvalidValue;
 
   int op, out_dt;
   GemmKArgs& k = plan->k;
@@ -569,7 +593,9 @@ hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan) {
   // Operands fit the LDS-DMA loader when both are K-contiguous with 16-byte
   // aligned rows and K is a multiple of 8; a compute tile's rows must stay
   // within a 2 GiB window of its buffer descriptor.
-  const bool dma_ok = a.stride_ak == 1 && a.stride_bk == 1 && (a.stride_am % 8) == 0 && (a.stride_bn % 8) == 0 &&
+  // (an fp32 launch arrives here with K and the operands' strides in 16-bit units: make_plan)
+  const int unit = a.ab_dtype == IRIS_DTYPE_F32 ? 2 : 1;
+  const bool dma_ok = a.stride_ak == unit && a.stride_bk == unit && (a.stride_am % 8) == 0 && (a.stride_bn % 8) == 0 &&
                       aligned16(a.a) && aligned16(a.b) && (a.K % 8) == 0 && a.stride_am > 0 && a.stride_bn > 0;
   auto fits = [&](const GemmKernelEntry& e) {
     if (!e.dma) return true;

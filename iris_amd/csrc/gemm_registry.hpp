@@ -10,10 +10,10 @@ namespace iris_amd {
 using GemmKernelFn = void (*)(const GemmKArgs);
 
 struct GemmKernelEntry {
-  int dt;      // operand type: IRIS_DTYPE_F16 | IRIS_DTYPE_BF16
+  int dt;      // operand type: IRIS_DTYPE_F16 | IRIS_DTYPE_BF16 | IRIS_DTYPE_F32
   int op;      // StoreOp
   int cm, cn;  // compute tile
-  int bk, wm, wn, stages;
+  int bk, wm, wn, stages;  // (bk in 16-bit units: half as many elements of fp32 operands)
   bool dma;    // LDS-DMA loader (needs K-contiguous, 16-byte aligned operands)
   bool splitk;  // the kernel can share a tile's K range with other programs
   bool split_owner;  // ... and its first part can add the others' partials itself (needed for stream-K runs)
@@ -160,7 +160,32 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 64, 64, 4, 1, 3, true, 4>, OP,                 \
                                                   IRIS_GEMM_ODT(DT, OP), true, false, true>(const GemmKArgs);
 
+// fp32 operands (fp32 output only): a short table.  The tiles are the 16-bit ones' (a stage of BK 16-bit units holds
+// BK / 2 elements of K; the names count elements); the matrix cores run fp32 at a sixteenth of the 16-bit rate, so any
+// tile that keeps them fed will do, and none is split along K or merged.
+template <class Cfg, int OP>
+constexpr GemmKernelEntry make_entry_f32(const char* name) {
+  static_assert(Cfg::DT == IRIS_DTYPE_F32 && (OP == OP_STORE32 || OP == OP_ATOMIC32), "fp32 operands, fp32 output");
+  return GemmKernelEntry{Cfg::DT, OP, Cfg::CM, Cfg::CN, Cfg::BK, Cfg::WM, Cfg::WN, Cfg::S, Cfg::DMA, false, false,
+                         Cfg::THREADS, Cfg::LW, Cfg::LDS_BYTES, &gemm_persistent_kernel<Cfg, OP, IRIS_DTYPE_F32, false>,
+                         nullptr, fused_fn<Cfg, OP, IRIS_DTYPE_F32>(), nullptr, nullptr, name};
+}
+#define IRIS_GEMM_F32_VARIANTS(X, OP)                                                   \
+  X(IRIS_DTYPE_F32, OP, 128, 128, 64, 2, 2, 4, true, 4, "128x128x32_w2x2_s4_f4_fp32")  \
+  X(IRIS_DTYPE_F32, OP, 128, 128, 64, 2, 2, 4, true, 0, "128x128x32_w2x2_s4_fp32")     \
+  X(IRIS_DTYPE_F32, OP, 64, 64, 64, 2, 2, 4, true, 0, "64x64x32_w2x2_s4_fp32")         \
+  X(IRIS_DTYPE_F32, OP, 64, 64, 32, 2, 2, 1, false, 0, "64x64x16_w2x2_generic_fp32")
+#define IRIS_GEMM_F32_ENTRY(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, NAME) \
+  make_entry_f32<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP>(NAME),
+#define IRIS_GEMM_F32_INSTANTIATE(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, NAME)                    \
+  template __global__ void gemm_persistent_kernel<GemmCfg<DT, CM, CN, BK, WM, WN, S, DMA, LW>, OP, \
+                                                  IRIS_DTYPE_F32, false>(const GemmKArgs);
+#define IRIS_GEMM_F32_INSTANTIATE_FUSED(DT, OP, CM, CN, BK, WM, WN, S, DMA, LW, NAME) \
+  IRIS_GEMM_INSTANTIATE_FUSED_##LW(DT, OP, CM, CN, BK, WM, WN, S, DMA)
+
 #define IRIS_GEMM_DECLARE(TAG) const GemmKernelEntry* gemm_entries_##TAG(int* count);
+IRIS_GEMM_DECLARE(f32_store32)
+IRIS_GEMM_DECLARE(f32_atomic32)
 IRIS_GEMM_DECLARE(bf16_store16)
 IRIS_GEMM_DECLARE(bf16_store32)
 IRIS_GEMM_DECLARE(bf16_atomic32)

@@ -141,8 +141,8 @@ def _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_s
     _require_cuda("b", b, device)
     if a.dtype != b.dtype:
         raise TypeError(f"a and b must share a dtype, got {a.dtype} and {b.dtype}")
-    if a.dtype not in (torch.float16, torch.bfloat16):
-        raise TypeError(f"operands must be fp16 or bf16, got {a.dtype}")
+    if a.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise TypeError(f"operands must be fp16, bf16 or fp32, got {a.dtype}")
     if BLK_M <= 0 or BLK_N <= 0 or gsize_m <= 0 or num_sms <= 0:
         raise ValueError("block sizes, gsize_m and the grid must be positive")
     total_tiles = cdiv(M, BLK_M) * cdiv(N, BLK_N)

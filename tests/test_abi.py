@@ -94,8 +94,12 @@ def test_launchers_reject_bad_arguments_without_a_device():
     g = _native.GemmArgs()  # all zero: no block sizes, no grid
     assert lib.iris_gemm_launch(ctypes.byref(g), None) == _native.HIP_ERROR_INVALID_VALUE
     g.block_m = g.block_n = g.group_size_m = g.num_sms = g.num_xcds = g.world_size = 1
-    g.ab_dtype = _native.DTYPE_F32  # operands must be 16-bit
+    g.ab_dtype = 7  # no such operand type
     assert lib.iris_gemm_launch(ctypes.byref(g), None) == _native.HIP_ERROR_INVALID_VALUE
+    g.ab_dtype, g.epilogue, g.c_global_dtype = _native.DTYPE_F32, _native.EPI_ALL_SCATTER, _native.DTYPE_BF16
+    g.c_global = 1024  # (never dereferenced: fp32 operands need an fp32 output, which the launcher checks first)
+    assert lib.iris_gemm_launch(ctypes.byref(g), None) == _native.HIP_ERROR_INVALID_VALUE
+    g.c_global, g.epilogue = None, 0
     g.ab_dtype = _native.DTYPE_BF16
     g.num_sms, g.num_xcds = 12, 8  # the XCD remap needs an even split
     assert lib.iris_gemm_launch(ctypes.byref(g), None) == _native.HIP_ERROR_INVALID_VALUE

@@ -39,6 +39,16 @@ def test_example_validates(tmp_path, example, extra):
     assert "Final C validation passed." in stdout and "registers used" in stdout
 
 
+@pytest.mark.parametrize("example", ["07_gemm_all_scatter", "08_gemm_atomics_all_reduce", "09_gemm_one_shot_all_reduce"])
+def test_example_validates_with_fp32_operands(tmp_path, example):
+    """``--datatype fp32`` of the reference scripts (09's benchmark.py:41-46): fp32 operands, fp32 C."""
+    data, stdout = run_example(tmp_path, example, "-m", "512", "-n", "384", "-k", "256", "--datatype", "fp32", "-v",
+                               "--virtual_ranks", "2")
+    assert data["success"] is True and data["world_size"] == 2
+    assert data["gemm_spills"] == 0
+    assert "Final C validation passed." in stdout
+
+
 def test_one_shot_example_with_virtual_ranks_and_benchmark(tmp_path):
     data, _ = run_example(tmp_path, "09_gemm_one_shot_all_reduce", "-m", "512", "-n", "512", "-k", "1024",
                           "--datatype", "fp16", "-v", "-b", "--virtual_ranks", "4", "--BLK_N", "128")
