@@ -72,6 +72,9 @@ def parse():
                     help="decoder workload: only this tile shape, as BLK_MxBLK_N (default: a sweep, and the "
                          "reference examples' default tile 256x64 beside it)")
     ap.add_argument("--shapes-gpus", default="1,2,4,8", help="shapes workload: the GPU counts the GEMMs are cut over")
+    ap.add_argument("--shapes-partial", default="operand", choices=["operand", "fp32"],
+                    help="shapes workload: element type of the one-shot producer's partial C: the operands' (what the "
+                         "reference's 09 script allocates, benchmark.py:103,124) or fp32 (twice the bytes)")
     ap.add_argument("--shapes-algorithms", default="all_scatter,one_shot",
                     help="shapes workload: all_scatter (N-shards) and / or one_shot (K-shards, the producer)")
     ap.add_argument("--workload", choices=["headline", "atomic", "decoder", "shapes", "fused"], default="headline",
@@ -557,7 +560,8 @@ def run_shapes(args, emit=True):
     """One rank's shard GEMM for every point of the reference's shape sweep, at the sweep's tile, beside the vendor
     library's plain GEMM on the same shard: the all-scatter ([8192, k] x [k, n / gpus], the tile stored into
     every rank's C behind its flag) and the producer of the one-shot all-reduce ([8192, k / gpus] x [k / gpus, n]
-    on K-shard views of the whole operands, an fp32 partial behind flags on the other ranks)."""
+    on K-shard views of the whole operands, a partial C of the operands' type behind flags on the other ranks, as
+    the reference's 09 script allocates it, benchmark.py:103,124; --shapes-partial fp32 for fp32 partials)."""
     import torch
 
     import iris_amd
@@ -567,7 +571,7 @@ def run_shapes(args, emit=True):
     gpus_list = [int(v) for v in args.shapes_gpus.split(",")]
     points = []
     for ws in gpus_list:
-        # per rank: A and B of the largest shape (0.6 + 0.5 GB), bf16 C, fp32 partial, flags
+        # per rank: A and B of the largest shape (0.6 + 0.5 GB), bf16 C, the partial, flags
         shmem = iris_amd.iris(2 << 30, virtual_ranks=ws)
         hb = shmem.get_heap_bases()
         xcds = ops.default_num_xcds(shmem.get_cu_count(), 256)
@@ -581,7 +585,7 @@ def run_shapes(args, emit=True):
             a.normal_(0, 0.02)
             bt.normal_(0, 0.02)
             cg = shmem.zeros((m, n), dtype=torch.bfloat16)
-            part = shmem.zeros((m, n), dtype=torch.float32)
+            part = shmem.zeros((m, n), dtype=torch.float32 if args.shapes_partial == "fp32" else torch.bfloat16)
             ns, ks = n // ws, k // ws
             for algorithm, (bm0, bn0, gsize_m) in zip(("all_scatter", "one_shot"), by_gpus[ws]):
                 if algorithm not in args.shapes_algorithms.split(","):
@@ -645,7 +649,8 @@ def run_shapes(args, emit=True):
         "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "dataset/mini.json's six GEMMs (m = 8192) cut over " + args.shapes_gpus + " GPUs at the "
                                "tiles of dataset/tiling.json, one rank's share on one GPU with the other ranks' "
-                               "heaps in the same HBM"},
+                               "heaps in the same HBM",
+                   "one_shot_partial": "fp32" if args.shapes_partial == "fp32" else "bf16 (the operands' type)"},
         "worst": ratios[0], "best": ratios[-1], "points": points}
     if emit:
         print(json.dumps(out))

@@ -387,9 +387,12 @@ def test_launcher_rejects_what_the_kernels_do_not_take(shmem):
     with pytest.raises(ValueError):  # fp16 result from bf16 operands
         ops.gemm_launch(a, b, None, shmem.zeros((64, 64), dtype=torch.float16), None, None, 0, 1, 4, 64, 64, 64, 1,
                         ops.EPI_ALL_SCATTER, notify=False)
-    with pytest.raises(TypeError):  # fp32 operands
+    with pytest.raises(ValueError):  # fp32 operands with a 16-bit result
         ops.gemm_launch(a.float(), b.float(), None, cg, None, None, 0, 1, 4, 64, 64, 64, 1, ops.EPI_ALL_SCATTER,
                         notify=False)
+    with pytest.raises(TypeError):  # integer operands
+        ops.gemm_launch(a.to(torch.int8), b.to(torch.int8), None, cg, None, None, 0, 1, 4, 64, 64, 64, 1,
+                        ops.EPI_ALL_SCATTER, notify=False)
 
 
 def test_small_tiles_get_two_programs_per_cu_when_the_launch_owns_the_device(shmem):
