@@ -1239,6 +1239,11 @@ gemm_persistent_kernel(const GemmKArgs p) {
   int peers_gone = 0;
   const GemmKArgs& p_outer = p;
   auto epilogue = [&]() __attribute__((always_inline)) {
+    if constexpr (PF) {
+      // (the prefetch hints' dwords land in this wave's scratch: all of them have, before the epilogue uses it;
+      // the last was issued pf_dist K-steps ago, so nothing is waited for in practice)
+      if (wave < 2) IRIS_WAIT_VMCNT(0);
+    }
     if (defer_publish && pending_tile >= 0) {
       // a one-step tile: the previous tile has not been published yet
       IRIS_WAIT_VMCNT(0);

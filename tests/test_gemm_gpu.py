@@ -150,6 +150,24 @@ def test_operands_the_dma_loader_cannot_take_use_the_generic_loader(shmem):
     assert float(cg3.float().abs().max()) == 0.0
 
 
+def test_a_launch_without_rows_or_columns_is_a_no_op(shmem):
+    """M == 0 or N == 0: nothing is launched, nothing is written, no flag moves (all three epilogues)."""
+    dtype = torch.bfloat16
+    A, B = make_ab(64, 64, 64, dtype)
+    a, b = to_heap(shmem, A), to_heap(shmem, B)
+    cg = shmem.full((64, 64), 5, dtype=dtype)
+    c = shmem.full((64, 64), 5, dtype=torch.float32)
+    flags = shmem.zeros((4,), dtype=torch.int32)
+    hb = shmem.get_heap_bases()
+    for av, bv in ((a[:0], b), (a, b[:, :0])):
+        ops.gemm_launch(av, bv, None, cg, flags, hb, 0, 1, 4, 64, 64, 64, 1, ops.EPI_ALL_SCATTER)
+        ops.gemm_launch(av, bv, None, cg, None, hb, 0, 1, 4, 64, 64, 64, 1, ops.EPI_ATOMIC_ADD)
+        ops.gemm_launch(av, bv, c, cg, flags, hb, 0, 1, 4, 64, 64, 64, 1, ops.EPI_ONE_SHOT, phase=ops.PHASE_PRODUCE)
+    torch.cuda.synchronize()
+    assert float((cg.float() - 5).abs().max()) == 0.0 and float((c - 5).abs().max()) == 0.0
+    assert flags.cpu().tolist() == [0] * 4
+
+
 def test_unaligned_and_strided_output(shmem):
     dtype = torch.bfloat16
     A, B = make_ab(256, 192, 64, dtype)
