@@ -181,6 +181,44 @@ def steady_ms(fn, settle_s=0.2, n=200):
     return s.elapsed_time(e) / n
 
 
+def shader_clock_mhz(fn, seconds=1.5):
+    """Median shader clock, as ``rocm-smi --showclocks`` reports it, while ``fn`` runs back to back on the GPU
+    (from a second thread; the first samples).  None where rocm-smi is missing or says nothing."""
+    import re
+    import subprocess
+    import threading
+
+    import torch
+
+    stop = threading.Event()
+
+    def keep_busy():
+        while not stop.is_set():
+            for _ in range(100):
+                fn()
+            torch.cuda.synchronize()
+
+    worker = threading.Thread(target=keep_busy)
+    worker.start()
+    samples = []
+    try:
+        time.sleep(0.5)  # (past the fast launches after an idle period)
+        t_end = time.perf_counter() + seconds
+        while time.perf_counter() < t_end:
+            try:
+                text = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
+            except (OSError, subprocess.SubprocessError):
+                break
+            m = re.search(r"sclk clock level: \S+ \((\d+)Mhz\)", text)
+            if m:
+                samples.append(int(m.group(1)))
+            time.sleep(0.1)
+    finally:
+        stop.set()
+        worker.join()
+    return int(statistics.median(samples)) if samples else None
+
+
 def graph_ms(fn, per_graph=20, replays=20, settle_s=0.02, batches=3):
     """Mean device ms per call of `fn`, with `per_graph` calls captured in a HIP
     graph so that the host's launch cost (tens of microseconds per call through
@@ -249,6 +287,15 @@ def context_figures(a, b, c_global, flops, gemm_on):
     ms = steady_ms(lambda: torch.matmul(az, bz, out=c_global))
     out["library_gemm_on_zeros"] = {"what": "torch.matmul (hipBLASLt), all-zero operands", "ms": round(ms, 5),
                                     "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
+    # The shader clock under each of the four: on zeros nothing holds it back; on data the board's power cap
+    # does, and the kernel that needs fewer clocks for the same work is held lower.
+    out["shader_clock_mhz"] = {
+        "how": "rocm-smi --showclocks sampled while the launch runs back to back, median",
+        "gemm": shader_clock_mhz(lambda: gemm_on(a, b)),
+        "library_gemm": shader_clock_mhz(lambda: torch.matmul(a, b, out=c_global)),
+        "gemm_on_zeros": shader_clock_mhz(lambda: gemm_on(az, bz)),
+        "library_gemm_on_zeros": shader_clock_mhz(lambda: torch.matmul(az, bz, out=c_global)),
+    }
     del az, bz
     groups, iters = 256, 4000
     sink = torch.empty(groups * 512, dtype=torch.float32, device="cuda")
@@ -1047,6 +1094,7 @@ def main():
             "library_gemm_on_zeros_ms": ctx["library_gemm_on_zeros"]["ms"],
             "mfma_only_tflops_on_such_data": ctx["mfma_sustained[random N(0,0.02)]"]["tflops"],
             "mfma_only_tflops_on_zeros": ctx["mfma_sustained[zeros]"]["tflops"],
+            "shader_clock_mhz": {k: v for k, v in ctx["shader_clock_mhz"].items() if k != "how"},
         }
 
     if args.copy_calibration:
