@@ -190,6 +190,9 @@ def shader_clock_mhz(fn, seconds=1.5):
 
     import torch
 
+    # (not under a profiler: its preloaded tool library would start up inside every rocm-smi child as well)
+    if "rocprofiler" in os.environ.get("LD_PRELOAD", "") or any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ):
+        return None
     stop = threading.Event()
 
     def keep_busy():
