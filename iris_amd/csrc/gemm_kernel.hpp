@@ -1201,6 +1201,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
   // (compiled into the 256 x 64 tile only: a test and a branch per K-step are felt by the small tiles, whose
   // steps take 0.2 us: [512,4096] x [4096,1376] in 64 x 64 x 128 tiles 19.9 -> 24.3 us)
   constexpr bool PF = Cfg::LW != 0 && Cfg::DMA && !FUSED && Cfg::CM == 256 && Cfg::CN == 64;
+  // a third build of the K-step, without the hand-over's tests (see `step`)
+  constexpr bool LEAN_STEPS = Cfg::DMA && !FUSED;
   __amdgpu_buffer_rsrc_t pf_rs = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, 0, 0x00020000);
   uint32_t pf_off = 0x80000000u;
   auto prefetch_setup = [&](const Item& it) __attribute__((always_inline)) {
@@ -1499,9 +1501,14 @@ gemm_persistent_kernel(const GemmKArgs p) {
     // too; what it fetches is never used (loads past the last step fetch
     // nothing).
     int ring_slot = 0;  // slot of the step about to run (rings whose depth is no power of two)
-    auto step = [&](int g, auto first_tag, auto par_tag) __attribute__((always_inline)) {
+    // LEAN: a step in the middle of a tile's K loop.  No tile waits to be published at its hand-over (the
+    // previous tile's flag went up at this tile's second hand-over) and the load cursor's next step lies inside
+    // the tile and is a full one, so the hand-over is a wait, the barrier and the refill, with no test between
+    // them: the waves all pass it at the same time, and what it costs, every SIMD's matrix core waits out.
+    auto step = [&](int g, auto first_tag, auto par_tag, auto lean_tag) __attribute__((always_inline)) {
       constexpr bool FIRST = decltype(first_tag)::value;
       constexpr int PAR = decltype(par_tag)::value;
+      constexpr bool LEAN = decltype(lean_tag)::value;
       int slot_g, slot_n;  // ring slots of steps g and g+1
       if constexpr (Cfg::S_POW2) {
         slot_g = g & (Cfg::S - 1);
@@ -1543,9 +1550,11 @@ gemm_persistent_kernel(const GemmKArgs p) {
         }
         // hand-over of stage g+1: wait for this wave's part of its slab
         // (S-2 younger slabs may stay in flight), then meet the other waves
-        const int pend = __builtin_amdgcn_readfirstlane(pending_tile);
-        const int skip = __builtin_amdgcn_readfirstlane(pending_skip);
-        if constexpr (Cfg::LW != 0) {
+        const int pend = LEAN ? -1 : __builtin_amdgcn_readfirstlane(pending_tile);
+        const int skip = LEAN ? 0 : __builtin_amdgcn_readfirstlane(pending_skip);
+        if constexpr (LEAN) {
+          if (Cfg::LW == 0 || fetcher) IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
+        } else if constexpr (Cfg::LW != 0) {
           if (fetcher) {
             IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
           } else if (pend >= 0 && skip == 0) {
@@ -1559,12 +1568,14 @@ gemm_persistent_kernel(const GemmKArgs p) {
           IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
         }
         block_barrier_raw();
-        if (pend >= 0) {
-          if (skip == 0) {
-            if (wave == 0) publish_tile<MERGED>(p, pend, lane);
-            pending_tile = -1;
-          } else {
-            pending_skip = 0;
+        if constexpr (!LEAN) {
+          if (pend >= 0) {
+            if (skip == 0) {
+              if (wave == 0) publish_tile<MERGED>(p, pend, lane);
+              pending_tile = -1;
+            } else {
+              pending_skip = 0;
+            }
           }
         }
         const IRIS_LDS char* nstage = lds + slot_n * Cfg::STAGE;
@@ -1594,8 +1605,13 @@ gemm_persistent_kernel(const GemmKArgs p) {
           // every wave is past its reads of stage g: refill it with step g+S
           if (fetcher) {
             ld.issue(p, rstage, l_k, fwave);
-            advance_load_cursor();
+            if constexpr (LEAN)
+              ++l_k;
+            else
+              advance_load_cursor();
           }
+        } else if constexpr (LEAN) {
+          ++l_k;
         } else {
           advance_load_cursor();
         }
@@ -1603,14 +1619,14 @@ gemm_persistent_kernel(const GemmKArgs p) {
     };
     // B buffer a step starts with: substeps alternate, so with an odd KSUB
     // it flips from step to step
-    auto run_step = [&](int g, auto first_tag) __attribute__((always_inline)) {
+    auto run_step = [&](int g, auto first_tag, auto lean_tag) __attribute__((always_inline)) {
       if constexpr (Cfg::KSUB % 2 == 0) {
-        step(g, first_tag, std::integral_constant<int, 0>{});
+        step(g, first_tag, std::integral_constant<int, 0>{}, lean_tag);
       } else {
         if (g & 1)
-          step(g, first_tag, std::integral_constant<int, 1>{});
+          step(g, first_tag, std::integral_constant<int, 1>{}, lean_tag);
         else
-          step(g, first_tag, std::integral_constant<int, 0>{});
+          step(g, first_tag, std::integral_constant<int, 0>{}, lean_tag);
       }
     };
     int g = 0;
@@ -1619,12 +1635,26 @@ gemm_persistent_kernel(const GemmKArgs p) {
       const KRange kr = k_range<Cfg, SPLIT>(p, sr, pid, it, nk);
       prefetch_setup(c_it);
       prefetch_step(kr.k_begin + p.pf_dist, kr.k_end);
-      run_step(g, std::true_type{});
+      run_step(g, std::true_type{}, std::false_type{});
       ++g;
       const int steps = kr.k_end - kr.k_begin;
-      for (int k = 1; k < steps; ++k, ++g) {
+      // Steps [2, lean_end) are lean: the previous tile was published at the second hand-over, and the load
+      // cursor, S steps ahead, moves on to a full step of this tile (the K loop's last step may be a partial one).
+      const int lean_end = LEAN_STEPS ? steps - Cfg::S - 1 - ((p.K % Cfg::BK) != 0 ? 1 : 0) : 0;
+      int k = 1;
+      for (; k < steps && k < 2; ++k, ++g) {
         prefetch_step(kr.k_begin + k + p.pf_dist, kr.k_end);
-        run_step(g, std::false_type{});
+        run_step(g, std::false_type{}, std::false_type{});
+      }
+      if constexpr (LEAN_STEPS) {
+        for (; k < lean_end; ++k, ++g) {
+          prefetch_step(kr.k_begin + k + p.pf_dist, kr.k_end);
+          run_step(g, std::false_type{}, std::true_type{});
+        }
+      }
+      for (; k < steps; ++k, ++g) {
+        prefetch_step(kr.k_begin + k + p.pf_dist, kr.k_end);
+        run_step(g, std::false_type{}, std::false_type{});
       }
       if constexpr (ONE_ITEM) IRIS_WAIT_VMCNT(0);  // (the loads past the last step fetch nothing, and nothing follows)
       epilogue();
