@@ -1201,7 +1201,8 @@ gemm_persistent_kernel(const GemmKArgs p) {
   // (compiled into the 256 x 64 tile only: a test and a branch per K-step are felt by the small tiles, whose
   // steps take 0.2 us: [512,4096] x [4096,1376] in 64 x 64 x 128 tiles 19.9 -> 24.3 us)
   constexpr bool PF = Cfg::LW != 0 && Cfg::DMA && !FUSED && Cfg::CM == 256 && Cfg::CN == 64;
-  // a third build of the K-step, without the hand-over's tests (see `step`)
+  // a third build of the K-step, without the hand-over's tests (see `step`; not with the reduce inside the program,
+  // where the K loop is the smaller part and a third copy of the step adds to what the 128-accumulator tiles spill)
   constexpr bool LEAN_STEPS = Cfg::DMA && !FUSED;
   __amdgpu_buffer_rsrc_t pf_rs = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, 0, 0x00020000);
   uint32_t pf_off = 0x80000000u;
