@@ -77,7 +77,7 @@ def parse():
                          "reference's 09 script allocates, benchmark.py:103,124) or fp32 (twice the bytes)")
     ap.add_argument("--shapes-algorithms", default="all_scatter,one_shot",
                     help="shapes workload: all_scatter (N-shards) and / or one_shot (K-shards, the producer)")
-    ap.add_argument("--workload", choices=["headline", "atomic", "decoder", "shapes", "fused"], default="headline",
+    ap.add_argument("--workload", choices=["headline", "atomic", "decoder", "shapes", "fused", "fp32"], default="headline",
                     help="headline: the 8192x8192x1024 shard GEMM + reduce (the metric's configuration); atomic: eight "
                          "K-shard GEMMs adding into one fp32 C; decoder: 6.7B-decoder-shaped shards for M in "
                          "{1,16,128,512,2048}; shapes: one rank's shard GEMM at every point of the reference's shape "
@@ -324,6 +324,62 @@ def context_figures(a, b, c_global, flops, gemm_on):
             "one_store_per_k_step_extra_us": round(t["one_store_per_k_step"] - t["none"], 1)}
         del region
     return out
+
+
+def run_fp32(args, emit=True):
+    """The headline shard with fp32 operands (the reference scripts' --datatype fp32): A[8192,1024] x B[1024,8192]
+    on K-shard views, fp32 C behind a flag per 256 x 256 tile, beside the vendor library's fp32 GEMM on the same
+    operands.  The matrix cores run fp32 at 157.3 TFLOP/s."""
+    import torch
+
+    import iris_amd
+    from iris_amd import ops
+
+    M = N = 8192
+    K, K_total = 1024, 8192
+    shmem = iris_amd.iris(2 << 30)
+    a_full = shmem.zeros((M, K_total), dtype=torch.float32)
+    bt_full = shmem.zeros((N, K_total), dtype=torch.float32)
+    a_full.normal_(0, 0.02)
+    bt_full.normal_(0, 0.02)
+    a, b = a_full[:, :K], bt_full[:, :K].T
+    cg = shmem.zeros((M, N), dtype=torch.float32)
+    flags = shmem.zeros((1024,), dtype=torch.int32)
+    lib = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    largs = (a, b, None, cg, flags, None, 0, 1, 256, 256, 256, 64, 4, ops.EPI_ALL_SCATTER)
+    kw = dict(num_xcds=ops.default_num_xcds(shmem.get_cu_count(), 256))
+
+    def ours():
+        ops.gemm_launch(*largs, **kw)
+
+    def library():
+        torch.matmul(a, b, out=lib)
+
+    ours()
+    library()
+    torch.cuda.synchronize()
+    err = (cg - lib).abs().max().item()
+    assert err <= 1e-4 * lib.abs().max().item(), f"fp32 GEMM differs from the library's by {err}"
+    assert flags.cpu().tolist() == [1] * 1024
+    flops = 2.0 * M * N * K
+    ms = steady_ms(ours, n=50)
+    lib_ms = steady_ms(library, n=50)
+    peak = 157.3
+    result = {
+        "metric": "shard GEMM + flag-published epilogue with fp32 operands", "value": round(flops / ms / 1e9, 2),
+        "unit": "TFLOP/s", "n_gpus": 1, "ms_per_step": round(ms, 5), "higher_is_better": True, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "fp32 A[8192,1024] x B[1024,8192] (K-shard views, lda=ldb=8192), 256x256 tiles -> fp32 "
+                               "in the fine-grained heap, one ready flag per tile", "grid": 256},
+        "kernel": ops.gemm_plan_name(*largs, **kw),
+        "roofline": {"bound": "mfma", "achieved": round(flops / ms / 1e9, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(flops / ms / 1e9 / peak, 4), "traffic": None},
+        "library_ms": round(lib_ms, 5), "library_tflops": round(flops / lib_ms / 1e9, 2),
+        "max_abs_diff_vs_library": err,
+    }
+    if emit:
+        print(json.dumps(result))
+    return result
 
 
 def run_atomic(args, emit=True):
@@ -907,6 +963,8 @@ def main():
         return run_decoder(args)
     if args.workload == "shapes":
         return run_shapes(args)
+    if args.workload == "fp32":
+        return run_fp32(args)
     if args.workload == "fused":
         return run_fused(args)
 
@@ -1122,6 +1180,7 @@ def main():
         args.shapes_gpus = "8"  # (the whole sweep, 1 to 8 GPUs, is the --workload shapes run)
         sweep = run_shapes(args, emit=False)
         fz = run_fused(args, emit=False)
+        f32 = run_fp32(args, emit=False)
         details["other_workloads"] = {
             "atomic_accumulate": {k: at[k] for k in ("value", "unit", "ms_per_step", "atomic_updates_per_s",
                                                      "atomic_ceiling", "config")},
@@ -1133,6 +1192,8 @@ def main():
                                               for pt in sweep["points"]]},
             "one_shot_in_program": {k: fz[k] for k in ("config", "in_program", "two_kernels",
                                                        "in_program_vs_two_kernels", "checked")},
+            "fp32_operands": {k: f32[k] for k in ("config", "kernel", "value", "unit", "ms_per_step", "roofline",
+                                                  "library_ms", "library_tflops")},
         }
         # one line each for the result line
         result["other_workloads"] = {
@@ -1146,6 +1207,8 @@ def main():
                                               "best": sweep["best"]},
             "one_shot_in_program_2_ranks_ms": fz["in_program"]["ms"],
             "one_shot_two_kernels_2_ranks_ms": fz["two_kernels"]["ms"],
+            "fp32_operands_tflops": f32["value"],
+            "fp32_operands_library_tflops": f32["library_tflops"],
         }
 
     if not args.no_cpu:
