@@ -139,6 +139,13 @@ struct GemmKArgs {
   // (MERGED builds) the launch covers the caller's columns of tiles from this one on: its flags sit that many
   // columns to the right in the caller's grid of flag_num_pid_m x flag_num_pid_n tiles
   int flag_pn_base;
+  // Staggered start (the unsplit eight-wave 256 x 256 tile; 0: none).  The CUs of an XCD that finish their tiles
+  // together send their 128 KiB of output stores each at the same moment, and a store that finds the XCD's write
+  // path full holds its wave at issue, with the next tile's first MFMAs behind it.  With stagger_groups > 1 the
+  // programs of an XCD start in that many groups, stagger_sleeps * 576 clocks apart, and stay that far apart for
+  // the whole launch (they all do the same work): two groups 2 us apart take 3 % off the headline launch on zeros
+  // and 1.5 % on data, the 2 us that the later group ends after the first included.
+  int stagger_groups, stagger_sleeps;
 };
 
 template <int DT>
@@ -1135,6 +1142,13 @@ gemm_persistent_kernel(const GemmKArgs p) {
     }
   }
 
+  if constexpr (Cfg::NW == 8 && Cfg::CM == 256 && Cfg::CN == 256 && !SPLIT && !FUSED) {
+    // (workgroups are dealt to the XCDs in turn: blockIdx.x / num_xcds counts a program's place on its XCD)
+    if (p.stagger_groups > 1) {
+      const int group = (blockIdx.x / p.num_xcds) % p.stagger_groups;
+      for (int i = 0; i < group * p.stagger_sleeps; ++i) __builtin_amdgcn_s_sleep(9);
+    }
+  }
   constexpr bool split = SPLIT;
   // The split build of a tile without the owner's hand-over only ever runs split-K proper (stream-K runs need
   // the owner's way): one (tile, part) item per program.  Saying so at compile time takes the item loop, the

@@ -266,6 +266,20 @@ void launch_constants(const iris_gemm_args& a, const GemmKernelEntry& pick, Gemm
   // long a stage takes to arrive from HBM ([8192,14336] x [14336,448] in 256 x 64 tiles: 175 -> 161 us eight
   // steps ahead, 155 sixteen ahead); the wider tiles' steps are bound by the matrix cores' power budget on real
   // data and gain nothing (256 x 128: 427 -> 440 us on N(0, 0.02) data, 408 -> 380 us on zeros).
+  // Staggered start (see GemmKArgs::stagger_groups): the unsplit eight-wave 256 x 256 tile, when every program has
+  // two tiles or more, so that there are epilogues whose store bursts the stagger keeps apart (a launch of one
+  // tile per program would only end later).  Two groups, 8 x 576 clocks = 2 us apart: [8192,1024] x [1024,8192]
+  // 90.2 -> 87.6 us on zeros, 113.7 -> 112.0 on N(0, 0.02) data; [8192,1536] x [1536,4096] stored to eight ranks
+  // 185.6 -> 182.6; [8192,7168] x [7168,4096] (two tiles a program, 112 K-steps each) unchanged.  Only for walks of
+  // at most 64 K-steps: on a long walk the epilogues are little beside the K loop, and programs that fetch the
+  // same panels two microseconds apart find less of them in their XCD's L2 ([8192,36864] x [36864,4608]: +2 %).
+  k.stagger_groups = k.stagger_sleeps = 0;
+  if (pick.cm == 256 && pick.cn == 256 && pick.wm * pick.wn == 8 && pick.fetch_waves == 0 && k.split_k == 1 &&
+      !k.stream_k && a.num_xcds > 1 && k.sub_m == 1 && k.sub_n == 1 && k.total_tiles >= 2 * (int64_t)a.num_sms &&
+      a.num_sms >= 2 * a.num_xcds && nk <= 64) {
+    k.stagger_groups = 2;
+    k.stagger_sleeps = 8;
+  }
   k.pf_dist = k.pf_sa = k.pf_sb = 0;
   const int pf_dist = 8;
   if (pick.fetch_waves > 0 && pick.cm == 256 && pick.cn == 64 && !k.stream_k && k.sub_m == 1 && k.sub_n == 1 && nk >= 16 * pf_dist &&
