@@ -124,6 +124,17 @@ int iris_hip_arch_name(int device, char* buf, size_t len);
 #define IRIS_GEMM_VARIANT_FEW_ROWS 1000
 #define IRIS_GEMM_VARIANT_PERSISTENT 1001
 
+/* iris_gemm_args.touch_ahead.  The eight-wave 256 x 256 tile has a build whose programs touch, one dword per 128-byte
+ * line, their share of the operand lines that the K-steps three ahead will load, so that the lines are in the
+ * XCD's L2 when the stage loads ask for them.  It pays where a round of tiles streams its operands from HBM (more
+ * bytes than the 256 MB last-level cache holds) and costs a few per cent where they are cache-resident: AUTO lets
+ * the launcher decide by the launch's bytes per round of tiles, ON takes the build wherever the picked tile has it
+ * (unsplit launches of that tile with a store epilogue on more than one XCD), OFF never.  The results are the same
+ * bits either way.  The reference has no counterpart (its loads are the Triton compiler's, gemm_*:170-199). */
+#define IRIS_GEMM_TOUCH_AUTO 0
+#define IRIS_GEMM_TOUCH_ON 1
+#define IRIS_GEMM_TOUCH_OFF 2
+
 /* Special value of iris_gemm_args.split_k: cut the launch's K-steps (all
  * tiles, in tile order) into num_sms equal runs that start and end anywhere
  * in a tile, the stream-K schedule the reference's wrappers describe and size
@@ -195,6 +206,7 @@ typedef struct iris_gemm_args {
    * are bit-identical. */
   int32_t split_handover;
   int32_t flag_sem;     /* IRIS_FLAG_SEM_*: how a tile's flag orders its data                    */
+  int32_t touch_ahead;  /* IRIS_GEMM_TOUCH_*                                                     */
 } iris_gemm_args;
 
 /*

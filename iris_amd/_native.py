@@ -31,6 +31,7 @@ SPLIT_STREAM_K = -1  # GemmArgs.split_k: stream-K
 HANDOVER_AUTO, HANDOVER_OWNER, HANDOVER_SLICED, HANDOVER_PAIR = 0, 1, 2, 3  # GemmArgs.split_handover
 # how a tile's flag orders its data (IRIS_FLAG_SEM_*)
 FLAG_SEM_WRITE_THROUGH, FLAG_SEM_RELEASE_ACQUIRE = 0, 1
+TOUCH_AUTO, TOUCH_ON, TOUCH_OFF = 0, 1, 2
 # status word (IRIS_STATUS_*)
 STATUS_OK, STATUS_SPIN_TIMEOUT = 0, 1
 
@@ -84,6 +85,7 @@ class GemmArgs(ctypes.Structure):
         ("split_k", ctypes.c_int32),
         ("split_handover", ctypes.c_int32),
         ("flag_sem", ctypes.c_int32),
+        ("touch_ahead", ctypes.c_int32),
     ]
 
 

@@ -187,13 +187,16 @@ struct Mfma<IRIS_DTYPE_F32> {
 // of fetch and multiply time.  LW_ = 4 adds one wave per SIMD that does
 // nothing but issue the stage loads and wait for them; the WM x WN waves then
 // issue no memory instruction in the K loop.
-template <int DT_, int CM_, int CN_, int BK_, int WM_, int WN_, int S_, bool DMA_, int LW_ = 0>
+template <int DT_, int CM_, int CN_, int BK_, int WM_, int WN_, int S_, bool DMA_, int LW_ = 0, bool TOUCH_ = false>
 struct GemmCfg {
   static constexpr int DT = DT_, CM = CM_, CN = CN_, BK = BK_, WM = WM_, WN = WN_, S = S_;
   static constexpr bool DMA = DMA_;
   static constexpr int NW = WM * WN, NT = NW * 64;  // the waves (threads) that multiply and store
   static constexpr int LW = LW_;
   static constexpr int NL = LW ? LW : NW;           // the waves that fetch
+  // TOUCH_: a build of the eight-wave 256 x 256 tile that touches lines of K-steps to come (see Loader::touch)
+  static constexpr bool TOUCH = TOUCH_;
+  static_assert(!TOUCH_ || (DMA_ && LW_ == 0 && WM_ * WN_ == 8 && CM_ == 256 && CN_ == 256), "the touching build's tile");
   static constexpr int THREADS = (NW + LW) * 64;    // launch size
   static constexpr int TM = CM / WM, TN = CN / WN;
   static constexpr int IM = TM / 16, IN = TN / 16;  // 16x16 MFMA blocks of the wave tile
@@ -370,6 +373,8 @@ struct Loader {
   uint32_t va, vb;
   int step_a, step_b;
   int k_limit;  // K
+  // (Cfg::TOUCH) byte offset of the row whose line this lane touches ahead of the loads, out of range for none
+  uint32_t ta, tb;
 
   // The chunk of the row that a lane fetches is the same for every load:
   // the swizzle period divides the rows between two loads of a wave.
@@ -397,7 +402,21 @@ struct Loader {
     vb = (uint32_t)(((int64_t)row * p.sbn + ck) * 2);
     step_a = (int)((int64_t)Cfg::NL * Cfg::RPB * p.sam * 2);
     step_b = (int)((int64_t)Cfg::NL * Cfg::RPB * p.sbn * 2);
+    if constexpr (Cfg::TOUCH) {
+      // this program's share of the panels' rows: `first`, `first + share`, ... (the shares are powers of two)
+      const int q = wave * 64 + lane;
+      const int row_a = ((it.n0 / Cfg::CN) & (p.pf_sa - 1)) + p.pf_sa * q;
+      const int row_b = ((it.m0 / Cfg::CM) & (p.pf_sb - 1)) + p.pf_sb * q;
+      ta = row_a < rows_a ? (uint32_t)((int64_t)row_a * p.sam * 2) : 0x80000000u;
+      tb = row_b < rows_b ? (uint32_t)((int64_t)row_b * p.sbn * 2) : 0x80000000u;
+    }
     before_step(k, wave, lane);
+  }
+  // Touch, with one dword per lane, this program's share of the lines of K-step `k` (two loads, always issued, so
+  // that the waits that follow count the same whether a lane has a row or not).  The dwords land in `scratch`.
+  __device__ inline void touch(IRIS_LDS char* scratch, int k) const {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (IRIS_LDS void*)scratch, 4, ta, k * Cfg::BK * 2, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (IRIS_LDS void*)scratch, 4, tb, k * Cfg::BK * 2, 0, 0);
   }
   // The load cursor is about to load step `k`: park the chunks past K.
   __device__ inline void before_step(int k, int wave, int lane) {
@@ -407,7 +426,10 @@ struct Loader {
   // The program has no more steps to load: the loads are still issued, so
   // that every K-step keeps the same number of loads in flight, but fetch
   // nothing.
-  __device__ inline void park() { va = vb = 0x80000000u; }
+  __device__ inline void park() {
+    va = vb = 0x80000000u;
+    if constexpr (Cfg::TOUCH) ta = tb = 0x80000000u;
+  }
 
   // Issue load `i` of K-step `k` into the stage at LDS address `stage`.  The
   // K offset rides in the scalar offset.
@@ -1218,6 +1240,10 @@ gemm_persistent_kernel(const GemmKArgs p) {
   // a third build of the K-step, without the hand-over's tests (see `step`; not with the reduce inside the program,
   // where the K loop is the smaller part and a third copy of the step adds to what the 128-accumulator tiles spill)
   constexpr bool LEAN_STEPS = Cfg::DMA && !FUSED;
+  // the lean steps of the eight-wave 256 x 256 tile each end with the two touches of Loader::touch, which the
+  // next lean step's hand-over leaves in flight
+  constexpr bool PF8 = Cfg::TOUCH && LEAN_STEPS;
+  constexpr int TOUCHES = PF8 ? 2 : 0;
   __amdgpu_buffer_rsrc_t pf_rs = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, 0, 0x00020000);
   uint32_t pf_off = 0x80000000u;
   auto prefetch_setup = [&](const Item& it) __attribute__((always_inline)) {
@@ -1568,7 +1594,7 @@ gemm_persistent_kernel(const GemmKArgs p) {
         const int pend = LEAN ? -1 : __builtin_amdgcn_readfirstlane(pending_tile);
         const int skip = LEAN ? 0 : __builtin_amdgcn_readfirstlane(pending_skip);
         if constexpr (LEAN) {
-          if (Cfg::LW == 0 || fetcher) IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
+          if (Cfg::LW == 0 || fetcher) IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2) + TOUCHES);
         } else if constexpr (Cfg::LW != 0) {
           if (fetcher) {
             IRIS_WAIT_VMCNT(Cfg::L * (Cfg::S - 2));
@@ -1661,7 +1687,19 @@ gemm_persistent_kernel(const GemmKArgs p) {
         prefetch_step(kr.k_begin + k + p.pf_dist, kr.k_end);
         run_step(g, std::false_type{}, std::false_type{});
       }
-      if constexpr (LEAN_STEPS) {
+      if constexpr (PF8) {
+        // every lean step is entered with the two touches issued last
+        if (k < lean_end) {
+          const int dist = p.pf_dist;
+          ld.touch(ws, min(l_k + dist, l_kend - 1));
+          for (;;) {
+            run_step(g, std::false_type{}, std::true_type{});
+            ++k, ++g;
+            if (k >= lean_end) break;
+            ld.touch(ws, min(l_k + dist, l_kend - 1));
+          }
+        }
+      } else if constexpr (LEAN_STEPS) {
         for (; k < lean_end; ++k, ++g) {
           prefetch_step(kr.k_begin + k + p.pf_dist, kr.k_end);
           run_step(g, std::false_type{}, std::true_type{});

@@ -300,6 +300,37 @@ void launch_constants(const iris_gemm_args& a, const GemmKernelEntry& pick, Gemm
       k.pf_sb = (int)rows;
     }
   }
+  // The same hints for the eight-wave 256 x 256 tile, whose every wave also loads: they are a build of their own
+  // (GemmKernelEntry::fn_touch), taken where a round of tiles streams its operands from HBM.  Looping
+  // [8192,14336] x [14336,2048] (294 MB of operands, one tile a program): 358 -> 339 us three steps ahead, 345 four,
+  // 352 eight (an XCD's share of eight steps, 3 MB, no longer stays in its 4 MB L2), 411 when every program touches
+  // all its lines instead of its share; on zeros 337 -> 296.  [8192,28672] x [28672,4096] (two tiles a program)
+  // 1393 -> 1344.  Where the operands stay in the 256 MB last-level cache the touches only add L2 requests:
+  // [8192,12288] x [12288,2048] (252 MB) +3 %, [8192,7168] x [7168,4096] +2 %; and an XCD whose tiles are two rows
+  // of sixteen (group size 2) fetches half as many lines again per step and is bound by that, not by latency
+  // ([8192,36864] x [36864,4608]: +5 %).  So: at least 272 MB of operands per round of tiles, and an XCD block of at
+  // least four tiles either way.
+  if (a.touch_ahead != IRIS_GEMM_TOUCH_OFF && pick.fn_touch && k.split_k == 1 && !k.stream_k && k.sub_m == 1 && k.sub_n == 1) {
+    const int64_t per_xcd = a.num_xcds > 1 ? (k.xcd_per > 0 ? k.xcd_per : (k.num_sms / a.num_xcds)) : k.num_sms;
+    const int g_rows = k.G < k.num_pid_m ? k.G : k.num_pid_m;
+    int64_t cols = per_xcd / (g_rows > 0 ? g_rows : 1);
+    if (cols < 1) cols = 1;
+    if (cols > k.num_pid_n) cols = k.num_pid_n;
+    int64_t rows = per_xcd / cols;
+    if (rows < 1) rows = 1;
+    // (the kernel takes its share of a panel's rows with a mask: powers of two)
+    int sa = 1, sb = 1;
+    while (sa * 2 <= cols && sa < 64) sa *= 2;
+    while (sb * 2 <= rows && sb < 64) sb *= 2;
+    const int64_t rounds = (k.total_tiles + k.num_sms - 1) / k.num_sms;
+    const int64_t operand_bytes = ((int64_t)a.M + a.N) * a.K * 2;
+    const bool streams = nk >= 32 && sa >= 4 && sb >= 4 && operand_bytes >= rounds * ((int64_t)272 << 20);
+    if (a.touch_ahead == IRIS_GEMM_TOUCH_ON || streams) {
+      k.pf_dist = 3;
+      k.pf_sa = sa;
+      k.pf_sb = sb;
+    }
+  }
 }
 
 // Validate `a` and build the launch plan.  Returns hipSuccess,
@@ -555,6 +586,8 @@ hipError_t make_plan_body(const iris_gemm_args& a, Plan* plan) {
       return hipErrorInvalidValue;
   }
   if (out_dt != IRIS_DTYPE_F32 && out_dt != a.ab_dtype) return hipErrorInvalidValue;
+  if (a.touch_ahead != IRIS_GEMM_TOUCH_AUTO && a.touch_ahead != IRIS_GEMM_TOUCH_ON && a.touch_ahead != IRIS_GEMM_TOUCH_OFF)
+    return hipErrorInvalidValue;
   if (a.flag_sem != IRIS_FLAG_SEM_WRITE_THROUGH && a.flag_sem != IRIS_FLAG_SEM_RELEASE_ACQUIRE)
     return hipErrorInvalidValue;
   if (k.flag_mode != 0 && a.flag_sem == IRIS_FLAG_SEM_RELEASE_ACQUIRE) k.flag_mode |= FLAG_RELEASE;
@@ -747,13 +780,21 @@ using namespace iris_amd;
 
 namespace {
 
+// Whether the plan's launch is the build that touches lines of K-steps to come (launch_constants decides; a
+// launch that splits K has no such build).
+bool plan_touches(const Plan& plan) {
+  const GemmKernelEntry* e = plan.entry;
+  return e && !plan.skinny && !plan.in_program && plan.k.split_k == 1 && !plan.k.stream_k && plan.k.pf_dist > 0 && e->fn_touch;
+}
+
 // The build of the picked kernel that the plan launches.
 GemmKernelFn plan_fn(const Plan& plan) {
   const GemmKernelEntry* e = plan.entry;
   if (plan.in_program) return e->fn_fused;
   const bool split = plan.k.split_k > 1 || plan.k.stream_k;
-  if (plan.remap_flags) return split ? e->fn_split_merged : e->fn_merged;
-  return split ? e->fn_split : e->fn;
+  const bool touch = plan_touches(plan);
+  if (plan.remap_flags) return split ? e->fn_split_merged : touch ? e->fn_touch_merged : e->fn_merged;
+  return split ? e->fn_split : touch ? e->fn_touch : e->fn;
 }
 
 // Enqueue what `plan` describes on `stream`.  (`args` is the caller's launch: only a reduce kernel behind the GEMM
@@ -967,6 +1008,10 @@ extern "C" int iris_gemm_plan_name(const iris_gemm_args* args, char* buf, size_t
                 : plan.k.merge_m * plan.k.merge_n == 4 ? "+four_tiles_each"
                 : plan.k.merge_m * plan.k.merge_n == 8 ? "+eight_tiles_each"
                                                        : "");
+  if (plan_touches(plan)) {
+    const size_t n = std::strlen(buf);
+    std::snprintf(buf + n, len > n ? len - n : 0, "+touch_ahead");
+  }
   if (plan.last_round) {
     const size_t n = std::strlen(buf);
     std::snprintf(buf + n, len > n ? len - n : 0, "+last_round_in_%d_parts", plan.k_last.split_k);

@@ -25,6 +25,8 @@ struct GemmKernelEntry {
   GemmKernelFn fn_fused;  // build with the one-shot reduce inside the program (store epilogues), or null
   GemmKernelFn fn_merged;  // build whose tiles are blocks of the caller's (store epilogues, 256 x 128 and 256 x 256), or null
   GemmKernelFn fn_split_merged;  // ... and its split-K build, or null
+  GemmKernelFn fn_touch;         // unsplit build that touches lines of K-steps to come (the eight-wave 256 x 256 tile), or null
+  GemmKernelFn fn_touch_merged;  // ... whose tiles are blocks of the caller's
   const char* name;
 };
 
@@ -69,13 +71,28 @@ constexpr GemmKernelFn split_merged_fn() {
     return nullptr;
 }
 
+// The eight-wave 256 x 256 tile's builds with the touches of Loader::touch (store epilogues).
+template <class Cfg>
+constexpr bool touch_build = Cfg::CM == 256 && Cfg::CN == 256 && Cfg::DMA && Cfg::BK == 64 && Cfg::LW == 0 && Cfg::NW == 8 &&
+                             Cfg::S == 2 && Cfg::WM == 2;
+template <int DT>
+using TouchCfg = GemmCfg<DT, 256, 256, 64, 2, 4, 2, true, 0, true>;
+template <class Cfg, int OP, int ODT, bool MERGED>
+constexpr GemmKernelFn touch_fn() {
+  if constexpr ((OP == OP_STORE16 || OP == OP_STORE32) && touch_build<Cfg>)
+    return &gemm_persistent_kernel<TouchCfg<Cfg::DT>, OP, ODT, false, false, MERGED>;
+  else
+    return nullptr;
+}
+
 template <class Cfg, int OP>
 constexpr GemmKernelEntry make_entry(const char* name) {
   constexpr int ODT = (OP == OP_STORE32 || OP == OP_ATOMIC32) ? IRIS_DTYPE_F32 : Cfg::DT;
   return GemmKernelEntry{Cfg::DT, OP,      Cfg::CM, Cfg::CN, Cfg::BK,        Cfg::WM,
                          Cfg::WN, Cfg::S,  Cfg::DMA, Cfg::SPLITK, Cfg::SPLIT_OWNER, Cfg::THREADS, Cfg::LW, Cfg::LDS_BYTES,
                          &gemm_persistent_kernel<Cfg, OP, ODT, false>, split_fn<Cfg, OP, ODT>(), fused_fn<Cfg, OP, ODT>(),
-                         merged_fn<Cfg, OP, ODT>(), split_merged_fn<Cfg, OP, ODT>(), name};
+                         merged_fn<Cfg, OP, ODT>(), split_merged_fn<Cfg, OP, ODT>(), touch_fn<Cfg, OP, ODT, false>(),
+                         touch_fn<Cfg, OP, ODT, true>(), name};
 }
 
 // The variants, in the launcher's order of preference: the first entry whose
@@ -158,7 +175,11 @@ constexpr GemmKernelEntry make_entry(const char* name) {
   template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 64, 64, 4, 1, 3, true, 4>, OP,                 \
                                                   IRIS_GEMM_ODT(DT, OP), false, false, true>(const GemmKArgs); \
   template __global__ void gemm_persistent_kernel<GemmCfg<DT, 256, 64, 64, 4, 1, 3, true, 4>, OP,                 \
-                                                  IRIS_GEMM_ODT(DT, OP), true, false, true>(const GemmKArgs);
+                                                  IRIS_GEMM_ODT(DT, OP), true, false, true>(const GemmKArgs);  \
+  template __global__ void gemm_persistent_kernel<TouchCfg<DT>, OP, IRIS_GEMM_ODT(DT, OP), false, false, false>(  \
+      const GemmKArgs);                                                                                           \
+  template __global__ void gemm_persistent_kernel<TouchCfg<DT>, OP, IRIS_GEMM_ODT(DT, OP), false, false, true>(   \
+      const GemmKArgs);
 
 // fp32 operands (fp32 output only): a short table.  The tiles are the 16-bit ones' (a stage of BK 16-bit units holds
 // BK / 2 elements of K; the names count elements); the matrix cores run fp32 at a sixteenth of the 16-bit rate, so any
@@ -168,7 +189,7 @@ constexpr GemmKernelEntry make_entry_f32(const char* name) {
   static_assert(Cfg::DT == IRIS_DTYPE_F32 && (OP == OP_STORE32 || OP == OP_ATOMIC32), "fp32 operands, fp32 output");
   return GemmKernelEntry{Cfg::DT, OP, Cfg::CM, Cfg::CN, Cfg::BK, Cfg::WM, Cfg::WN, Cfg::S, Cfg::DMA, false, false,
                          Cfg::THREADS, Cfg::LW, Cfg::LDS_BYTES, &gemm_persistent_kernel<Cfg, OP, IRIS_DTYPE_F32, false>,
-                         nullptr, fused_fn<Cfg, OP, IRIS_DTYPE_F32>(), nullptr, nullptr, name};
+                         nullptr, fused_fn<Cfg, OP, IRIS_DTYPE_F32>(), nullptr, nullptr, nullptr, nullptr, name};
 }
 #define IRIS_GEMM_F32_VARIANTS(X, OP)                                                   \
   X(IRIS_DTYPE_F32, OP, 128, 128, 64, 2, 2, 4, true, 4, "128x128x32_w2x2_s4_f4_fp32")  \

@@ -35,6 +35,9 @@ from ._native import (
     HANDOVER_PAIR,
     FLAG_SEM_WRITE_THROUGH,
     FLAG_SEM_RELEASE_ACQUIRE,
+    TOUCH_AUTO,
+    TOUCH_ON,
+    TOUCH_OFF,
 )
 
 __all__ = [
@@ -61,6 +64,9 @@ __all__ = [
     "SCOPE_SYSTEM",
     "FLAG_SEM_WRITE_THROUGH",
     "FLAG_SEM_RELEASE_ACQUIRE",
+    "TOUCH_AUTO",
+    "TOUCH_ON",
+    "TOUCH_OFF",
 ]
 
 _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
@@ -234,8 +240,13 @@ def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size,
                 gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, scope=SCOPE_AGENT, variant=0,
                 mm_begin_timestamp=None, mm_end_timestamp=None, status=None, spin_timeout_ticks=0, partials=None,
                 locks=None, split_k=0, noalloc=False, split_handover=HANDOVER_AUTO,
-                flag_sem=FLAG_SEM_WRITE_THROUGH):
+                flag_sem=FLAG_SEM_WRITE_THROUGH, touch_ahead=TOUCH_AUTO):
     """Launch the persistent shard GEMM ``a @ b`` with a tile-publishing epilogue.
+
+    ``touch_ahead``: ``TOUCH_AUTO`` lets the launcher decide whether the
+    256 x 256 tile runs the build that touches the operand lines of K-steps to
+    come (it does where a round of tiles streams more bytes than the last-level
+    cache holds), ``TOUCH_ON`` / ``TOUCH_OFF`` force the choice; same bits.
 
     ``flag_sem``: ``FLAG_SEM_WRITE_THROUGH`` (write-through stores, then a
     relaxed flag add: validated with concurrent producers and consumers on one
@@ -278,6 +289,7 @@ def gemm_launch(a, b, c, c_global, tile_completed, heap_bases, rank, world_size,
         launch = _native.lib().iris_gemm_launch
     args.split_handover = split_handover
     args.flag_sem = flag_sem
+    args.touch_ahead = touch_ahead
     stream = torch.cuda.current_stream(a.device).cuda_stream
     with torch.cuda.device(a.device):
         err = launch(ctypes.byref(args), stream)
@@ -306,11 +318,12 @@ def gemm_split_k(a, b, c, c_global, tile_completed, heap_bases, rank, world_size
 
 def gemm_plan_name(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N, BLK_K,
                    gsize_m, epilogue, *, phase=PHASE_FUSED, notify=True, num_xcds=1, variant=0, partials=None,
-                   locks=None, split_k=0):
+                   locks=None, split_k=0, touch_ahead=TOUCH_AUTO):
     """Name of the kernel a launch with these arguments would run."""
     args = _fill_gemm_args(a, b, c, c_global, tile_completed, heap_bases, rank, world_size, num_sms, BLK_M, BLK_N,
                            BLK_K, gsize_m, epilogue, phase, notify, num_xcds, SCOPE_AGENT, variant, None, None, None,
                            0, partials, locks, split_k)
+    args.touch_ahead = touch_ahead
     buf = ctypes.create_string_buffer(128)
     with torch.cuda.device(a.device):
         err = _native.lib().iris_gemm_plan_name(ctypes.byref(args), buf, 128)
