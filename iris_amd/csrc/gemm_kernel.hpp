@@ -135,6 +135,9 @@ struct GemmKArgs {
   // one dword of its share of the lines that step k + pf_dist will need (every pf_sa-th row of A, every pf_sb-th
   // of B: the launch's tiles per XCD in either direction), so that the stage loads find them in L2.  Nothing
   // depends on the loaded values.
+  // The touching build of the eight-wave 256 x 256 tile (GemmCfg::TOUCH) reads the same three: its touches are
+  // issued by every wave, last in a K-step, for the step pf_dist beyond the load cursor (see Loader::touch), and
+  // the shares are powers of two there.
   int pf_dist, pf_sa, pf_sb;
   // (MERGED builds) the launch covers the caller's columns of tiles from this one on: its flags sit that many
   // columns to the right in the caller's grid of flag_num_pid_m x flag_num_pid_n tiles
@@ -412,8 +415,12 @@ struct Loader {
     }
     before_step(k, wave, lane);
   }
-  // Touch, with one dword per lane, this program's share of the lines of K-step `k` (two loads, always issued, so
-  // that the waits that follow count the same whether a lane has a row or not).  The dwords land in `scratch`.
+  // Touch, with one dword per lane, this program's share of the lines of K-step `k`, so that they are on their way
+  // from HBM into the XCD's L2 before the stage loads of that step ask for them.  Two loads, one per operand,
+  // always issued (a lane without a row holds an offset out of range), so that the waits that follow count the
+  // same in every wave.  Loads return in order: the K-step issues them after its stage loads, and the next
+  // hand-over leaves exactly these two in flight.  The dwords land in `scratch` (LDS that nothing reads inside a
+  // K loop), not in a register, which the compiler would hand on before the load has returned.
   __device__ inline void touch(IRIS_LDS char* scratch, int k) const {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (IRIS_LDS void*)scratch, 4, ta, k * Cfg::BK * 2, 0, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (IRIS_LDS void*)scratch, 4, tb, k * Cfg::BK * 2, 0, 0);
