@@ -1712,6 +1712,29 @@ gemm_persistent_kernel(const GemmKArgs p) {
           run_step(g, std::false_type{}, std::true_type{});
         }
       }
+      if constexpr (LEAN_STEPS && !PF8) {
+        // Step lean_end is the one in which the load cursor crosses into the next tile (decode, loader set-up).
+        // The S steps behind it load that tile's first steps and are lean again, when those are full steps and
+        // the cursor does not cross a second time (behind the program's last tile it is parked on [0, nk)).
+        if (k == lean_end && k < steps && (p.K % Cfg::BK) == 0) {
+          int next_steps = nk;
+          if constexpr (SPLIT) {
+            if (it + 1 < n_items) {
+              const KRange nr = k_range<Cfg, SPLIT>(p, sr, pid, it + 1, nk);
+              next_steps = nr.k_end - nr.k_begin;
+            }
+          }
+          prefetch_step(kr.k_begin + k + p.pf_dist, kr.k_end);
+          run_step(g, std::false_type{}, std::false_type{});
+          ++k, ++g;
+          if (next_steps > Cfg::S) {
+            for (; k < steps; ++k, ++g) {
+              prefetch_step(kr.k_begin + k + p.pf_dist, kr.k_end);
+              run_step(g, std::false_type{}, std::true_type{});
+            }
+          }
+        }
+      }
       for (; k < steps; ++k, ++g) {
         prefetch_step(kr.k_begin + k + p.pf_dist, kr.k_end);
         run_step(g, std::false_type{}, std::false_type{});
