@@ -37,8 +37,8 @@ PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E, published
 # WRITE_SIZE runs of this script, each scaled by what the same counter reads for the --copy-calibration
 # kernel (profiles/gemm_all_scatter_bf16_8192x8192x1024.txt, profiles/one_shot_reduce_fp32x8_8192x8192.txt).
 # Counters cannot be read from inside a run, so these are carried here and dropped for non-default variants.
-GEMM_TRAFFIC_BYTES = 333128636
-REDUCE_TRAFFIC_BYTES = 2280894251
+GEMM_TRAFFIC_BYTES = 335108222
+REDUCE_TRAFFIC_BYTES = 2280882394
 
 M, N, K_SHARD, K_TOTAL = 8192, 8192, 1024, 8192
 BLK_M, BLK_N, BLK_K, GSIZE_M, GRID = 256, 256, 64, 4, 256
